@@ -1,0 +1,90 @@
+/*
+ * C ABI of libgemm.so: FP8 (OCP e4m3fn) blockwise-scaled GEMM for MI355X (gfx950).
+ *
+ *   C[m,n] = bf16( sum_kb  a_scale[m,kb] * b_scale[n/128,kb] * sum_{k in block kb} A[m,k] * B[n,k] )
+ *
+ * Memory layouts are the reference launcher's (tests/gemm/gemm_test.cpp:82-98, task.yml:22-27):
+ *   a   fp8 e4m3fn bytes, [K][M]   (element (m,k) at a[k*M + m])
+ *   b   fp8 e4m3fn bytes, [K][N]   (element (n,k) at b[k*N + n])
+ *   as  fp32,             [K/128][M]
+ *   bs  fp32,             [K/128][ceil(N/128)]
+ *   c   bf16,             [M][N] row-major, fully overwritten
+ * All pointers are device pointers. K must be a positive multiple of 128; M, N >= 1.
+ * Shapes with M%16==0, N%16==0 and 16-byte aligned a/b/c take the tiled MFMA path; anything
+ * else takes a slower bounds-checked kernel (the role of the reference's legacy kernel,
+ * src/gemm/gemm_kernel_legacy.cpp:237-374).
+ * Not thread-safe across host threads (one lazily grown workspace per process), like the reference.
+ */
+#ifndef RF_GEMM_H
+#define RF_GEMM_H
+
+#include <stddef.h>
+#include "metrics.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#ifndef HIP_INCLUDE_HIP_HIP_RUNTIME_API_H
+typedef struct ihipStream_t *hipStream_t;
+#endif
+
+/* Status codes of the rf_* entry points. */
+enum {
+    RF_OK = 0,
+    RF_ERR_BAD_SHAPE = 1,      /* m<1, n<1, k<128 or k%128 != 0 */
+    RF_ERR_NULL_POINTER = 2,
+    RF_ERR_HIP = 3,            /* a HIP call failed; see rf_gemm_last_error() */
+    RF_ERR_BAD_CONFIG = 4      /* explicit config not available for this shape */
+};
+
+/* One launch plan: which kernel variant and how K is split.
+ * Replaces a DISPATCH_GEMM(...) line of the reference (src/gemm/gemm_launcher.cpp:158-162,229-259). */
+typedef struct rf_gemm_config {
+    int variant;      /* index into the variant table, see rf_gemm_variant_info(); -1 = bounds-checked kernel */
+    int split_k;      /* >= 1; K blocks are divided over this many partial sums */
+    int group_m;      /* tile-order grouping along M for L2 reuse (>=1) */
+} rf_gemm_config;
+
+/* Drop-in for the reference's launcher entry (src/gemm/gemm_launcher.cpp:182-184):
+ * same name, argument order and behaviour: enqueues on job_stream0 and returns; on any error prints a
+ * message and abort()s (src/gemm/gemm_launcher.cpp:96-100,261-264). metrics may be NULL; if not,
+ * entries[0].time (ms) and entries[0].gflops are written from a stream callback once the work has
+ * finished (src/utils/timer.cpp:12-60). */
+void run(void *a, void *b, void *as, void *bs, void *c, int m, int n, int k, PerfMetrics *metrics,
+         hipStream_t job_stream0);
+
+/* Same computation, returns a status instead of aborting. Replaces launch_gemm / launch_gemm_legacy
+ * (src/gemm/gemm_launcher.cpp:43-101,104-148) with shape-generic dispatch. */
+int rf_fp8_gemm(const void *a, const void *b, const float *as, const float *bs, void *c,
+                int m, int n, int k, hipStream_t stream);
+
+/* As rf_fp8_gemm with an explicit plan (cfg == NULL selects automatically). This is what the tuner
+ * drives instead of recompiling a template per configuration (tuner/template/gemm_perf.cpp:21-38). */
+int rf_fp8_gemm_ex(const void *a, const void *b, const float *as, const float *bs, void *c,
+                   int m, int n, int k, const rf_gemm_config *cfg, hipStream_t stream);
+
+/* The plan rf_fp8_gemm would use for (m,n,k) on the current device: the gfx950 replacement of the
+ * per-shape table in src/gemm/gemm_launcher.cpp:229-259 / tuner/gemm_tuner.py. */
+int rf_gemm_select_config(int m, int n, int k, rf_gemm_config *out);
+
+/* Variant table introspection (for the tuner and tests). Returns RF_ERR_BAD_CONFIG past the end. */
+int rf_gemm_num_variants(void);
+int rf_gemm_variant_info(int variant, int *block_m, int *block_n, int *waves_m, int *waves_n, int *lds_bytes);
+
+/* Device workspace (split-K partial sums) needed for a shape under the automatic plan, in bytes. */
+size_t rf_gemm_workspace_bytes(int m, int n, int k);
+
+/* Optional explicit set-up / tear-down of the process-wide workspace on the current device. run() and
+ * rf_fp8_gemm() grow it lazily on first use (the reference's init_workspace, src/gemm/gemm_launcher.cpp:30-36,50-53,
+ * allocates a fixed 1.5 GB instead). rf_gemm_init(bytes) pre-allocates so that later calls allocate nothing. */
+int rf_gemm_init(size_t workspace_bytes);
+void rf_gemm_destroy(void);
+
+/* Text of the last failure on this thread's most recent rf_* call ("" if none). */
+const char *rf_gemm_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

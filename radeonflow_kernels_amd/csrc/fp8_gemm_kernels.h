@@ -1,0 +1,316 @@
+// Device kernels of the FP8 (OCP e4m3fn) blockwise-scaled GEMM for gfx950 (MI355X).
+//
+// Replaces the reference's transpose + rocWMMA pipeline (src/gemm/transpose_kernel.cpp:17-63,
+// src/gemm/gemm_kernel.cpp:306-562, src/gemm/gemm_kernel.cpp:288-303) with a design built on
+// three gfx950 features:
+//   * global_load_lds_dwordx4  - 16 B per lane straight from HBM/L2 into LDS, no VGPR staging;
+//   * ds_read_b64_tr_b8        - LDS transpose read: a 16-lane group that points at 8 k-rows x 16
+//                                bytes gets back, per lane, 8 consecutive k for one m (or n). The
+//                                operands arrive M-/N-contiguous ([K][M], [K][N]) and MFMA wants
+//                                K-contiguous bytes per lane, so this removes the reference's two
+//                                transpose pre-passes entirely;
+//   * v_mfma_f32_16x16x128_f8f6f4 - one MFMA consumes exactly one 128-wide scale block.
+//
+// Data flow per workgroup: a BM x BN output tile, K walked in blocks of 128. Each K block is one
+// LDS stage holding A[k0:k0+128][m0:m0+BM] and B[k0:k0+128][n0:n0+BN] exactly as they lie in
+// memory (rows of BM / BN bytes), with the 16-byte chunks of every row XOR-swizzled so that the
+// transpose reads are bank-conflict free. Two stages are double-buffered.
+//
+// MFMA orientation: the B-matrix fragment is the MFMA "A" operand (rows = n) and the A-matrix
+// fragment is the MFMA "B" operand (columns = m). A lane (L = lane%16, g = lane/16) then holds
+// D[n = 4g..4g+3][m = L]: four consecutive n of one row m, i.e. 8 contiguous bytes of bf16 C, and
+// needs a single scale a_scale[m,kb]*b_scale[nb,kb] per 16x16 tile.
+//
+// Numerics (what the reference's kernel does, src/gemm/gemm_kernel.cpp:138-208): the products of a
+// 128-K block are summed inside the MFMA in fp32 starting from zero, then acc = fma(sa*sb, partial, acc).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace rf {
+
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int BK = 128;        // K per stage == the quantisation block
+constexpr int NUM_XCD = 8;
+
+#define RF_LDS __attribute__((address_space(3)))
+#define RF_GLOBAL __attribute__((address_space(1)))
+
+// XOR applied to the 16-byte-chunk index of LDS row k (row width W bytes). Chosen so that the 32
+// lanes the LDS serves together in a transpose read (two 16-lane groups: 8 k-rows x 2 half-chunks
+// each, the groups 32 rows apart) touch all 64 banks exactly once.
+template <int W>
+__device__ __forceinline__ int swizzle_of_row(int k) {
+    constexpr int r = (W == 256) ? 0 : (W == 128) ? 1 : 2;   // log2(rows per 256 B bank wrap)
+    static_assert(W == 256 || W == 128 || W == 64, "tile row width");
+    return ((k & 7) >> r) | (((k >> 5) & 1) << (3 - r));
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    f32x2 v = {lo, hi};
+    bf16x2 h = __builtin_convertvector(v, bf16x2);           // v_cvt_pk_bf16_f32: RNE, NaN-safe
+    return __builtin_bit_cast(uint32_t, h);
+}
+
+// Workgroup id -> (tile_m, tile_n). Workgroups are dealt round-robin to the 8 XCDs (each with its
+// own L2), so id%8 is the XCD. Give every XCD a contiguous range of logical tile ids, and order
+// logical ids in groups of `group_m` tile rows so that the tiles resident on one XCD at a time
+// form a compact patch that re-uses A rows and B columns from that XCD's L2.
+__device__ __forceinline__ void tile_of_block(int bid, int nblocks, int tiles_m, int tiles_n, int group_m,
+                                              int &tile_m, int &tile_n) {
+    int xcd = bid % NUM_XCD, idx = bid / NUM_XCD;
+    int per = nblocks / NUM_XCD, rem = nblocks % NUM_XCD;
+    int id = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    int group_sz = group_m * tiles_n;
+    int grp = id / group_sz;
+    int first_m = grp * group_m;
+    int rows = tiles_m - first_m < group_m ? tiles_m - first_m : group_m;
+    int in_grp = id - grp * group_sz;
+    tile_m = first_m + in_grp % rows;
+    tile_n = in_grp / rows;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Tiled MFMA kernel. PARTIAL=false: writes bf16 C. PARTIAL=true: writes fp32 partial sums of the
+// K range of split blockIdx.y to ws[split][M][N].
+// Requirements checked by the host: M%16==0, N%16==0, M>=16, N>=16, a/b 16-byte aligned,
+// c 8-byte aligned, K%128==0.
+// ---------------------------------------------------------------------------------------------
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool PARTIAL>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_tile(
+    const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
+    const float *__restrict__ SB, void *__restrict__ Cout, int M, int N, int K, int kb_per_split,
+    int tiles_m, int tiles_n, int group_m) {
+    constexpr int NW = WAVES_M * WAVES_N;
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+    constexpr int TM = WM / 16, TN = WN / 16;
+    constexpr int STAGE_A = BK * BM, STAGE_B = BK * BN, STAGE = STAGE_A + STAGE_B;
+    constexpr int INST_A = STAGE_A / 1024 / NW, INST_B = STAGE_B / 1024 / NW;   // 1 KiB per wave instruction
+    static_assert(STAGE_A % (1024 * NW) == 0 && STAGE_B % (1024 * NW) == 0, "loads must divide evenly over waves");
+    static_assert(WN <= 128 && 128 % WN == 0, "a wave's N range must sit inside one scale block");
+    constexpr int CPR_A = BM / 16, CPR_B = BN / 16;          // 16-byte chunks per LDS row
+    constexpr int RPI_A = 1024 / BM, RPI_B = 1024 / BN;      // rows per load instruction
+
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int L = lane & 15, g = lane >> 4;
+    const int wm = wave % WAVES_M, wn = wave / WAVES_M;
+
+    int tile_m, tile_n;
+    tile_of_block(blockIdx.x, tiles_m * tiles_n, tiles_m, tiles_n, group_m, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int QK = K / BK, QN = (N + 127) / 128;
+    const int kb_begin = blockIdx.y * kb_per_split;
+    const int kb_end = kb_begin + kb_per_split < QK ? kb_begin + kb_per_split : QK;
+
+    // ---- global -> LDS: per-lane source offsets inside one K block (rows k_local, swizzled chunk) ----
+    uint32_t goff_a[INST_A], goff_b[INST_B];
+#pragma unroll
+    for (int i = 0; i < INST_A; i++) {
+        int q = wave * INST_A + i;
+        int kl = q * RPI_A + lane / CPR_A;
+        int c = (lane % CPR_A) ^ swizzle_of_row<BM>(kl);
+        int m = m0 + c * 16;
+        if (m + 16 > M) m = M - 16;                           // rows past M: any valid bytes will do
+        goff_a[i] = (uint32_t)kl * (uint32_t)M + (uint32_t)m;
+    }
+#pragma unroll
+    for (int i = 0; i < INST_B; i++) {
+        int q = wave * INST_B + i;
+        int kl = q * RPI_B + lane / CPR_B;
+        int c = (lane % CPR_B) ^ swizzle_of_row<BN>(kl);
+        int n = n0 + c * 16;
+        if (n + 16 > N) n = N - 16;
+        goff_b[i] = (uint32_t)kl * (uint32_t)N + (uint32_t)n;
+    }
+    auto issue_stage = [&](int stage, int kb) {
+        const uint8_t *ak = A + (size_t)kb * BK * M;
+        const uint8_t *bk = B + (size_t)kb * BK * N;
+        uint8_t *sa_lds = lds + stage * STAGE;
+        uint8_t *sb_lds = sa_lds + STAGE_A;
+#pragma unroll
+        for (int i = 0; i < INST_A; i++)
+            __builtin_amdgcn_global_load_lds((const RF_GLOBAL void *)(ak + goff_a[i]),
+                                             (RF_LDS void *)(sa_lds + (wave * INST_A + i) * 1024), 16, 0, 0);
+#pragma unroll
+        for (int i = 0; i < INST_B; i++)
+            __builtin_amdgcn_global_load_lds((const RF_GLOBAL void *)(bk + goff_b[i]),
+                                             (RF_LDS void *)(sb_lds + (wave * INST_B + i) * 1024), 16, 0, 0);
+    };
+
+    // ---- LDS -> MFMA operands: per-lane byte offsets of the transpose reads (stage 0, t = 0) ----
+    // lane (L,g) of read t points at row k = 32g + 8t + L/2, half (L&1) of 16-byte chunk c.
+    const int krow = 32 * g + (L >> 1);
+    uint32_t aoff[TM], boff[TN];
+    {
+        const int sw = swizzle_of_row<BM>(krow);              // independent of t (8t leaves k&7 and k>>5 alone)
+#pragma unroll
+        for (int j = 0; j < TM; j++)
+            aoff[j] = krow * BM + (((wm * TM + j) ^ sw) << 4) + 8 * (L & 1);
+    }
+    {
+        const int sw = swizzle_of_row<BN>(krow);
+#pragma unroll
+        for (int i = 0; i < TN; i++)
+            boff[i] = STAGE_A + krow * BN + (((wn * TN + i) ^ sw) << 4) + 8 * (L & 1);
+    }
+
+    // ---- scales: lane needs a_scale[kb][m] for its column m of every m-tile, and one b_scale ----
+    int srow[TM];
+#pragma unroll
+    for (int j = 0; j < TM; j++) {
+        int m = m0 + wm * WM + 16 * j + L;
+        srow[j] = m < M ? m : M - 1;
+    }
+    int nb = (n0 + wn * WN) >> 7;
+    if (nb > QN - 1) nb = QN - 1;
+
+    f32x4 acc[TM][TN];
+#pragma unroll
+    for (int j = 0; j < TM; j++)
+#pragma unroll
+        for (int i = 0; i < TN; i++) acc[j][i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    float sa_next[TM], sb_next;
+    auto load_scales = [&](int kb) {
+#pragma unroll
+        for (int j = 0; j < TM; j++) sa_next[j] = SA[(size_t)kb * M + srow[j]];
+        sb_next = SB[(size_t)kb * QN + nb];
+    };
+
+    if (kb_begin < kb_end) {
+        issue_stage(0, kb_begin);
+        load_scales(kb_begin);
+    }
+    for (int kb = kb_begin, it = 0; kb < kb_end; ++kb, ++it) {
+        // my loads for this stage have landed; after the barrier everyone's have, and everyone has
+        // finished reading the other stage (computed in the previous iteration)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        float s[TM];
+#pragma unroll
+        for (int j = 0; j < TM; j++) s[j] = sa_next[j] * sb_next;
+        if (kb + 1 < kb_end) {
+            issue_stage((it + 1) & 1, kb + 1);
+            load_scales(kb + 1);
+        }
+        const uint32_t sbase = (it & 1) * STAGE;
+        i32x8 bfrag[TN];
+#pragma unroll
+        for (int i = 0; i < TN; i++) {
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                i32x2 v = __builtin_amdgcn_ds_read_tr8_b64_v2i32((RF_LDS i32x2 *)(lds + sbase + boff[i] + t * 8 * BN));
+                bfrag[i][2 * t] = v[0];
+                bfrag[i][2 * t + 1] = v[1];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < TM; j++) {
+            i32x8 afrag;
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                i32x2 v = __builtin_amdgcn_ds_read_tr8_b64_v2i32((RF_LDS i32x2 *)(lds + sbase + aoff[j] + t * 8 * BM));
+                afrag[2 * t] = v[0];
+                afrag[2 * t + 1] = v[1];
+            }
+#pragma unroll
+            for (int i = 0; i < TN; i++) {
+                f32x4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bfrag[i], afrag, (f32x4){0.f, 0.f, 0.f, 0.f},
+                                                                          0, 0, 0, 0, 0, 0);
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[j][i][e] = __builtin_fmaf(s[j], p[e], acc[j][i][e]);
+            }
+        }
+    }
+
+    // ---- epilogue: lane holds C[m][n..n+3] per tile ----
+#pragma unroll
+    for (int j = 0; j < TM; j++) {
+        const int m = m0 + wm * WM + 16 * j + L;
+#pragma unroll
+        for (int i = 0; i < TN; i++) {
+            const int n = n0 + wn * WN + 16 * i + 4 * g;
+            if (m < M && n < N) {
+                if constexpr (PARTIAL) {
+                    float *ws = (float *)Cout + ((size_t)blockIdx.y * M + m) * N + n;
+                    *(f32x4 *)ws = acc[j][i];
+                } else {
+                    uint16_t *c = (uint16_t *)Cout + (size_t)m * N + n;
+                    uint2 v;
+                    v.x = pack_bf16x2(acc[j][i][0], acc[j][i][1]);
+                    v.y = pack_bf16x2(acc[j][i][2], acc[j][i][3]);
+                    *(uint2 *)c = v;
+                }
+            }
+        }
+    }
+}
+
+// Sum of split-K partials in split order 0..S-1, then one bf16 rounding
+// (the reference's reduce_kernel, src/gemm/gemm_kernel.cpp:288-303). 4 outputs per thread.
+__global__ __launch_bounds__(256) void reduce_splitk_bf16(const float *__restrict__ ws, uint16_t *__restrict__ C,
+                                                          size_t mn, int splits) {
+    size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= mn) return;
+    f32x4 s = *(const f32x4 *)(ws + i);
+    for (int p = 1; p < splits; p++) {
+        f32x4 v = *(const f32x4 *)(ws + (size_t)p * mn + i);
+        s[0] += v[0]; s[1] += v[1]; s[2] += v[2]; s[3] += v[3];
+    }
+    uint2 o;
+    o.x = pack_bf16x2(s[0], s[1]);
+    o.y = pack_bf16x2(s[2], s[3]);
+    *(uint2 *)(C + i) = o;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Bounds-checked kernel for shapes or alignments the tiled kernel does not take (M or N not a
+// multiple of 16, unaligned pointers). One wave per 16x16 output tile, bytes gathered directly
+// from global memory; out-of-range rows/columns contribute zeros and are not stored.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void gemm_fp8_blockscale_checked(
+    const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
+    const float *__restrict__ SB, uint16_t *__restrict__ C, int M, int N, int K) {
+    const int lane = threadIdx.x, L = lane & 15, g = lane >> 4;
+    const int m0 = blockIdx.y * 16, n0 = blockIdx.x * 16;
+    const int QK = K / BK, QN = (N + 127) / 128;
+    const int m_ld = m0 + L, n_ld = n0 + L;                  // operand rows this lane gathers
+    const bool m_ok = m_ld < M, n_ok = n_ld < N;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int kb = 0; kb < QK; kb++) {
+        union { i32x8 v; uint8_t b[32]; } fa, fb;
+#pragma unroll
+        for (int j = 0; j < 32; j++) {
+            size_t k = (size_t)kb * BK + 32 * g + j;
+            fa.b[j] = m_ok ? A[k * M + m_ld] : (uint8_t)0;
+            fb.b[j] = n_ok ? B[k * N + n_ld] : (uint8_t)0;
+        }
+        f32x4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb.v, fa.v, (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+        // lane holds D[n = n0+4g+e][m = m0+L]
+        float sa = m_ok ? SA[(size_t)kb * M + m_ld] : 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            int n = n0 + 4 * g + e;
+            float sb = n < N ? SB[(size_t)kb * QN + (n >> 7)] : 0.f;
+            acc[e] = __builtin_fmaf(sa * sb, p[e], acc[e]);
+        }
+    }
+    if (m_ok) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            int n = n0 + 4 * g + e;
+            if (n < N) C[(size_t)m_ld * N + n] = (uint16_t)(pack_bf16x2(acc[e], 0.f) & 0xffff);
+        }
+    }
+}
+
+}  // namespace rf

@@ -1,0 +1,326 @@
+// Host side of libgemm.so: the C ABI declared in include/rf_gemm.h.
+//
+// Takes the place of the reference's launcher (src/gemm/gemm_launcher.cpp): `run` keeps its
+// signature and abort-on-error behaviour; dispatch is shape-generic (a heuristic over a small
+// variant table tuned for gfx950) instead of a switch over 29 hard-coded shapes, and no transpose
+// pre-pass or transposed copies exist.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../../include/rf_gemm.h"
+#include "fp8_gemm_kernels.h"
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const std::string &msg) {
+    g_last_error = msg;
+    return code;
+}
+#define RF_HIP(expr)                                                                                   \
+    do {                                                                                               \
+        hipError_t e_ = (expr);                                                                        \
+        if (e_ != hipSuccess)                                                                          \
+            return fail(RF_ERR_HIP, std::string(#expr) + ": " + hipGetErrorString(e_));               \
+    } while (0)
+
+// ---- variant table -------------------------------------------------------------------------
+typedef void (*tile_kernel_t)(const uint8_t *, const uint8_t *, const float *, const float *, void *, int, int, int,
+                              int, int, int, int);
+struct Variant {
+    int bm, bn, waves_m, waves_n;
+    tile_kernel_t direct, partial;
+    int lds_bytes() const { return 2 * rf::BK * (bm + bn); }
+    int threads() const { return waves_m * waves_n * 64; }
+};
+#define RF_VARIANT(BM, BN, WM, WN)                                                         \
+    Variant { BM, BN, WM, WN, rf::gemm_fp8_blockscale_tile<BM, BN, WM, WN, false>,         \
+              rf::gemm_fp8_blockscale_tile<BM, BN, WM, WN, true> }
+const Variant kVariants[] = {
+    RF_VARIANT(256, 256, 2, 4),   // 0: 8 waves, wave tile 128(m) x 64(n), 128 KiB LDS
+    RF_VARIANT(128, 128, 2, 2),   // 1: 4 waves, wave tile 64 x 64, 64 KiB LDS (2 workgroups per CU)
+    RF_VARIANT(256, 128, 2, 2),   // 2: 4 waves, wave tile 128 x 64, 96 KiB LDS
+    RF_VARIANT(128, 256, 2, 4),   // 3: 8 waves, wave tile 64 x 64, 96 KiB LDS
+    RF_VARIANT(128, 64, 2, 1),    // 4: 2 waves, wave tile 64 x 64, 48 KiB LDS (3 workgroups per CU)
+};
+constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
+
+// ---- process-wide state ---------------------------------------------------------------------
+struct State {
+    std::mutex mu;
+    float *ws = nullptr;
+    size_t ws_bytes = 0;
+    bool attrs_set = false;
+    int num_cu = 0;
+    std::vector<std::pair<hipEvent_t, hipEvent_t>> free_events;
+};
+State &state() {
+    static State s;
+    return s;
+}
+
+int ensure_device_info(State &s) {
+    if (s.attrs_set) return RF_OK;
+    int dev = 0;
+    RF_HIP(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    RF_HIP(hipGetDeviceProperties(&prop, dev));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(RF_ERR_HIP, std::string("libgemm.so is built for gfx950 only, device is ") + prop.gcnArchName);
+    s.num_cu = prop.multiProcessorCount;
+    for (const Variant &v : kVariants) {
+        RF_HIP(hipFuncSetAttribute((const void *)v.direct, hipFuncAttributeMaxDynamicSharedMemorySize, v.lds_bytes()));
+        RF_HIP(hipFuncSetAttribute((const void *)v.partial, hipFuncAttributeMaxDynamicSharedMemorySize, v.lds_bytes()));
+    }
+    s.attrs_set = true;
+    return RF_OK;
+}
+
+int ensure_workspace(State &s, size_t bytes) {
+    if (bytes <= s.ws_bytes) return RF_OK;
+    if (s.ws) {
+        RF_HIP(hipDeviceSynchronize());      // earlier launches may still read the old buffer
+        RF_HIP(hipFree(s.ws));
+        s.ws = nullptr;
+        s.ws_bytes = 0;
+    }
+    RF_HIP(hipMalloc((void **)&s.ws, bytes));
+    s.ws_bytes = bytes;
+    return RF_OK;
+}
+
+inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+bool tiled_path_ok(const void *a, const void *b, const void *c, int m, int n) {
+    return m >= 16 && n >= 16 && m % 16 == 0 && n % 16 == 0 && ((uintptr_t)a % 16) == 0 && ((uintptr_t)b % 16) == 0 &&
+           ((uintptr_t)c % 8) == 0;
+}
+
+// Heuristic plan. Inputs: shape and CU count. The numbers come from sweeps on MI355X (256 CUs).
+void select_config(int m, int n, int k, int num_cu, bool tiled_ok, rf_gemm_config *out) {
+    out->split_k = 1;
+    out->group_m = 8;
+    if (!tiled_ok) {
+        out->variant = -1;
+        return;
+    }
+    const int qk = k / rf::BK;
+    int best = 1;
+    long tiles_big = (long)ceil_div(m, 256) * ceil_div(n, 256);
+    if (tiles_big >= num_cu) best = 0;
+    out->variant = best;
+    const Variant &v = kVariants[best];
+    long tiles = (long)ceil_div(m, v.bm) * ceil_div(n, v.bn);
+    long slots = (long)num_cu * (best == 1 ? 2 : 1);
+    if (tiles < slots && qk >= 4) {
+        int s = (int)(slots / tiles);
+        if (s > 8) s = 8;
+        while (s > 1 && qk / s < 2) s--;
+        out->split_k = s < 1 ? 1 : s;
+    }
+}
+
+int launch(const void *a, const void *b, const float *as, const float *bs, void *c, int m, int n, int k,
+           const rf_gemm_config *user_cfg, hipStream_t stream) {
+    g_last_error.clear();
+    if (m < 1 || n < 1 || k < rf::BK || k % rf::BK != 0)
+        return fail(RF_ERR_BAD_SHAPE, "unsupported shape M=" + std::to_string(m) + " N=" + std::to_string(n) +
+                                          " K=" + std::to_string(k) + " (need M,N>=1, K a positive multiple of 128)");
+    if (!a || !b || !as || !bs || !c) return fail(RF_ERR_NULL_POINTER, "null device pointer");
+    State &s = state();
+    std::lock_guard<std::mutex> lock(s.mu);
+    int rc = ensure_device_info(s);
+    if (rc != RF_OK) return rc;
+
+    const bool tiled_ok = tiled_path_ok(a, b, c, m, n);
+    rf_gemm_config cfg;
+    if (user_cfg) {
+        cfg = *user_cfg;
+        if (cfg.variant >= kNumVariants || cfg.variant < -1 || cfg.split_k < 1 || cfg.group_m < 1 ||
+            cfg.split_k > k / rf::BK || (cfg.variant >= 0 && !tiled_ok) || (cfg.variant < 0 && cfg.split_k != 1))
+            return fail(RF_ERR_BAD_CONFIG, "configuration not usable for this shape");
+    } else {
+        select_config(m, n, k, s.num_cu, tiled_ok, &cfg);
+    }
+
+    if (cfg.variant < 0) {
+        dim3 grid(ceil_div(n, 16), ceil_div(m, 16));
+        hipLaunchKernelGGL(rf::gemm_fp8_blockscale_checked, grid, dim3(64), 0, stream, (const uint8_t *)a,
+                           (const uint8_t *)b, as, bs, (uint16_t *)c, m, n, k);
+        RF_HIP(hipGetLastError());
+        return RF_OK;
+    }
+
+    const Variant &v = kVariants[cfg.variant];
+    const int tiles_m = ceil_div(m, v.bm), tiles_n = ceil_div(n, v.bn);
+    const int qk = k / rf::BK;
+    const int kb_per_split = ceil_div(qk, cfg.split_k);
+    const int splits = ceil_div(qk, kb_per_split);          // every split owns at least one K block
+    dim3 grid(tiles_m * tiles_n, splits);
+    dim3 block(v.threads());
+    if (splits == 1) {
+        hipLaunchKernelGGL(v.direct, grid, block, v.lds_bytes(), stream, (const uint8_t *)a, (const uint8_t *)b, as, bs,
+                           c, m, n, k, kb_per_split, tiles_m, tiles_n, cfg.group_m);
+        RF_HIP(hipGetLastError());
+    } else {
+        const size_t mn = (size_t)m * n;
+        rc = ensure_workspace(s, mn * splits * sizeof(float));
+        if (rc != RF_OK) return rc;
+        hipLaunchKernelGGL(v.partial, grid, block, v.lds_bytes(), stream, (const uint8_t *)a, (const uint8_t *)b, as,
+                           bs, (void *)s.ws, m, n, k, kb_per_split, tiles_m, tiles_n, cfg.group_m);
+        RF_HIP(hipGetLastError());
+        hipLaunchKernelGGL(rf::reduce_splitk_bf16, dim3((unsigned)((mn / 4 + 255) / 256)), dim3(256), 0, stream,
+                           (const float *)s.ws, (uint16_t *)c, mn, splits);
+        RF_HIP(hipGetLastError());
+    }
+    return RF_OK;
+}
+
+// ---- timing record for run() ----------------------------------------------------------------
+struct TimerJob {
+    hipEvent_t start, stop;
+    double flop;
+    float *time_ms, *gflops;
+};
+void timer_callback(hipStream_t, hipError_t status, void *user) {
+    TimerJob *job = static_cast<TimerJob *>(user);
+    if (status == hipSuccess) {
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, job->start, job->stop) == hipSuccess) {
+            if (job->time_ms) *job->time_ms = ms;
+            if (job->gflops) *job->gflops = (float)(job->flop / (ms * 1e-3) / 1e9);
+        }
+    }
+    State &s = state();
+    {
+        std::lock_guard<std::mutex> lock(s.mu);
+        s.free_events.emplace_back(job->start, job->stop);   // recycled, unlike the reference's growing list
+    }
+    delete job;
+}
+
+}  // namespace
+
+extern "C" {
+
+int rf_fp8_gemm(const void *a, const void *b, const float *as, const float *bs, void *c, int m, int n, int k,
+                hipStream_t stream) {
+    return launch(a, b, as, bs, c, m, n, k, nullptr, stream);
+}
+
+int rf_fp8_gemm_ex(const void *a, const void *b, const float *as, const float *bs, void *c, int m, int n, int k,
+                   const rf_gemm_config *cfg, hipStream_t stream) {
+    return launch(a, b, as, bs, c, m, n, k, cfg, stream);
+}
+
+int rf_gemm_select_config(int m, int n, int k, rf_gemm_config *out) {
+    g_last_error.clear();
+    if (!out) return fail(RF_ERR_NULL_POINTER, "out is null");
+    if (m < 1 || n < 1 || k < rf::BK || k % rf::BK != 0) return fail(RF_ERR_BAD_SHAPE, "unsupported shape");
+    State &s = state();
+    std::lock_guard<std::mutex> lock(s.mu);
+    int rc = ensure_device_info(s);
+    if (rc != RF_OK) return rc;
+    select_config(m, n, k, s.num_cu, m >= 16 && n >= 16 && m % 16 == 0 && n % 16 == 0, out);
+    return RF_OK;
+}
+
+int rf_gemm_num_variants(void) { return kNumVariants; }
+
+int rf_gemm_variant_info(int variant, int *block_m, int *block_n, int *waves_m, int *waves_n, int *lds_bytes) {
+    if (variant < 0 || variant >= kNumVariants) return RF_ERR_BAD_CONFIG;
+    const Variant &v = kVariants[variant];
+    if (block_m) *block_m = v.bm;
+    if (block_n) *block_n = v.bn;
+    if (waves_m) *waves_m = v.waves_m;
+    if (waves_n) *waves_n = v.waves_n;
+    if (lds_bytes) *lds_bytes = v.lds_bytes();
+    return RF_OK;
+}
+
+size_t rf_gemm_workspace_bytes(int m, int n, int k) {
+    rf_gemm_config cfg;
+    if (rf_gemm_select_config(m, n, k, &cfg) != RF_OK || cfg.variant < 0 || cfg.split_k <= 1) return 0;
+    const int qk = k / rf::BK;
+    const int kb_per_split = ceil_div(qk, cfg.split_k);
+    return (size_t)m * n * sizeof(float) * ceil_div(qk, kb_per_split);
+}
+
+int rf_gemm_init(size_t workspace_bytes) {
+    g_last_error.clear();
+    State &s = state();
+    std::lock_guard<std::mutex> lock(s.mu);
+    int rc = ensure_device_info(s);
+    if (rc != RF_OK) return rc;
+    return ensure_workspace(s, workspace_bytes);
+}
+
+void rf_gemm_destroy(void) {
+    State &s = state();
+    std::lock_guard<std::mutex> lock(s.mu);
+    if (s.ws) {
+        (void)hipDeviceSynchronize();
+        (void)hipFree(s.ws);
+    }
+    s.ws = nullptr;
+    s.ws_bytes = 0;
+    for (auto &p : s.free_events) {
+        (void)hipEventDestroy(p.first);
+        (void)hipEventDestroy(p.second);
+    }
+    s.free_events.clear();
+}
+
+const char *rf_gemm_last_error(void) { return g_last_error.c_str(); }
+
+void run(void *a, void *b, void *as, void *bs, void *c, int m, int n, int k, PerfMetrics *metrics,
+         hipStream_t job_stream0) {
+    TimerJob *job = nullptr;
+    if (metrics) {
+        job = new TimerJob();
+        State &s = state();
+        {
+            std::lock_guard<std::mutex> lock(s.mu);
+            if (!s.free_events.empty()) {
+                job->start = s.free_events.back().first;
+                job->stop = s.free_events.back().second;
+                s.free_events.pop_back();
+            } else {
+                job->start = job->stop = nullptr;
+            }
+        }
+        if (!job->start && (hipEventCreate(&job->start) != hipSuccess || hipEventCreate(&job->stop) != hipSuccess)) {
+            fprintf(stderr, "run: hipEventCreate failed\n");
+            abort();
+        }
+        job->flop = 2.0 * m * n * k;
+        job->time_ms = &metrics->entries[0].time;
+        job->gflops = &metrics->entries[0].gflops;
+        if (hipEventRecord(job->start, job_stream0) != hipSuccess) {
+            fprintf(stderr, "run: hipEventRecord failed\n");
+            abort();
+        }
+    }
+    int rc = launch(a, b, (const float *)as, (const float *)bs, c, m, n, k, nullptr, job_stream0);
+    if (rc != RF_OK) {
+        if (rc == RF_ERR_BAD_SHAPE) printf("Error: Unsupported shape M=%d, K=%d, N=%d\n", m, k, n);
+        fprintf(stderr, "Kernel execution failed.\n%s\n", g_last_error.c_str());
+        abort();
+    }
+    if (job) {
+        if (hipEventRecord(job->stop, job_stream0) != hipSuccess ||
+            hipStreamAddCallback(job_stream0, timer_callback, job, 0) != hipSuccess) {
+            fprintf(stderr, "run: could not enqueue the timing callback\n");
+            abort();
+        }
+    }
+}
+
+}  // extern "C"

@@ -1,0 +1,146 @@
+"""Host-side mirror of the reference's Python operator boundary, over the C ABI of libgemm.so.
+
+Mirrors the torch extension the reference generates (scripts/gen_submission.py:248-262,327-330):
+  fp8_mm(a, b, a_scale, b_scale, c)   m=a.size(0), n=b.size(0), k=a.size(1); current stream; run(...)
+  custom_kernel(data) -> c
+Tensors carry the reference's strides: a [m,k] and b [n,k] are transposed views of [K][M] / [K][N]
+fp8 storage, a_scale [m,k/128] and b_scale [ceil(n/128),k/128] are transposed views of [QK][M] /
+[QK][QN] fp32 storage, c is contiguous bf16 [m,n]. PyTorch is used for device memory and streams only.
+There is no CPU or PyTorch fallback: a missing library or a non-GPU tensor raises.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libgemm.so")
+_lib = None
+
+RF_OK = 0
+
+
+class GemmConfig(ctypes.Structure):
+    _fields_ = [("variant", ctypes.c_int), ("split_k", ctypes.c_int), ("group_m", ctypes.c_int)]
+
+    def __repr__(self):
+        return "GemmConfig(variant=%d, split_k=%d, group_m=%d)" % (self.variant, self.split_k, self.group_m)
+
+
+class PerfMetricEntry(ctypes.Structure):
+    _fields_ = [("name", ctypes.c_char * 20), ("time", ctypes.c_float), ("gflops", ctypes.c_float)]
+
+
+class PerfMetrics(ctypes.Structure):
+    _fields_ = [("count", ctypes.c_int), ("entries", PerfMetricEntry * 20)]
+
+
+EXPORTS = ("run", "rf_fp8_gemm", "rf_fp8_gemm_ex", "rf_gemm_select_config", "rf_gemm_num_variants",
+           "rf_gemm_variant_info", "rf_gemm_workspace_bytes", "rf_gemm_init", "rf_gemm_destroy",
+           "rf_gemm_last_error")
+
+
+def lib():
+    """Loads libgemm.so (built by radeonflow_kernels_amd.build). Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("libgemm.so is missing at %s: build it with `python -m radeonflow_kernels_amd.build`"
+                               % LIB_PATH)
+        L = ctypes.CDLL(LIB_PATH)
+        vp, i32 = ctypes.c_void_p, ctypes.c_int
+        L.run.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, ctypes.POINTER(PerfMetrics), vp]
+        L.run.restype = None
+        L.rf_fp8_gemm.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, vp]
+        L.rf_fp8_gemm.restype = i32
+        L.rf_fp8_gemm_ex.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, ctypes.POINTER(GemmConfig), vp]
+        L.rf_fp8_gemm_ex.restype = i32
+        L.rf_gemm_select_config.argtypes = [i32, i32, i32, ctypes.POINTER(GemmConfig)]
+        L.rf_gemm_select_config.restype = i32
+        L.rf_gemm_num_variants.restype = i32
+        L.rf_gemm_variant_info.argtypes = [i32] + [ctypes.POINTER(i32)] * 5
+        L.rf_gemm_variant_info.restype = i32
+        L.rf_gemm_workspace_bytes.argtypes = [i32, i32, i32]
+        L.rf_gemm_workspace_bytes.restype = ctypes.c_size_t
+        L.rf_gemm_init.argtypes = [ctypes.c_size_t]
+        L.rf_gemm_init.restype = i32
+        L.rf_gemm_destroy.restype = None
+        L.rf_gemm_last_error.restype = ctypes.c_char_p
+        _lib = L
+    return _lib
+
+
+def last_error():
+    return lib().rf_gemm_last_error().decode()
+
+
+def _check_layout(a, b, a_scale, b_scale, c):
+    if not (a.is_cuda and b.is_cuda and a_scale.is_cuda and b_scale.is_cuda and c.is_cuda):
+        raise ValueError("fp8_mm needs GPU tensors")
+    m, k = a.shape
+    n = b.shape[0]
+    qk, qn = k // 128, (n + 127) // 128
+    if a.element_size() != 1 or b.element_size() != 1:
+        raise ValueError("a and b must be 1-byte fp8 (e4m3fn) tensors")
+    if b.shape[1] != k or tuple(a_scale.shape) != (m, qk) or tuple(b_scale.shape) != (qn, qk) or tuple(c.shape) != (m, n):
+        raise ValueError("inconsistent shapes")
+    if a_scale.dtype != torch.float32 or b_scale.dtype != torch.float32 or c.dtype != torch.bfloat16:
+        raise ValueError("scales must be fp32 and c bf16")
+    # the launcher reads [K][M], [K][N], [QK][M], [QK][QN] storage: the tensors must be transposed views of that
+    def colmajor(t):
+        r, cdim = t.shape
+        return (t.stride(0) == 1 or r == 1) and (t.stride(1) == r or cdim == 1)
+    if not (colmajor(a) and colmajor(b) and colmajor(a_scale) and colmajor(b_scale) and c.is_contiguous()):
+        raise ValueError("a, b, a_scale, b_scale must be column-major (transposed views), c row-major contiguous")
+    return m, n, k
+
+
+def fp8_mm(a, b, a_scale, b_scale, c, config=None):
+    """c[m,n] = bf16(sum_kb a_scale*b_scale * (A_kb . B_kb^T)) on the current HIP stream; returns None."""
+    m, n, k = _check_layout(a, b, a_scale, b_scale, c)
+    stream = ctypes.c_void_p(torch.cuda.current_stream(a.device).cuda_stream)
+    L = lib()
+    cfg = ctypes.byref(config) if config is not None else None
+    with torch.cuda.device(a.device):
+        rc = L.rf_fp8_gemm_ex(a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(), c.data_ptr(),
+                              m, n, k, cfg, stream)
+    if rc != RF_OK:
+        raise RuntimeError("rf_fp8_gemm failed (%d): %s" % (rc, last_error()))
+
+
+def custom_kernel(data):
+    """The contest entry point: data = (a, b, a_scale, b_scale, c); returns c."""
+    a, b, a_scale, b_scale, c = data
+    fp8_mm(a, b, a_scale, b_scale, c)
+    return c
+
+
+def run_with_metrics(a, b, a_scale, b_scale, c):
+    """Calls the drop-in `run` entry with a PerfMetrics record; returns (time_ms, gflops) after a sync."""
+    m, n, k = _check_layout(a, b, a_scale, b_scale, c)
+    pm = PerfMetrics()
+    stream = ctypes.c_void_p(torch.cuda.current_stream(a.device).cuda_stream)
+    with torch.cuda.device(a.device):
+        lib().run(a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(), c.data_ptr(), m, n, k,
+                  ctypes.byref(pm), stream)
+        torch.cuda.synchronize(a.device)
+    return pm.entries[0].time, pm.entries[0].gflops, pm.count
+
+
+def select_config(m, n, k):
+    cfg = GemmConfig()
+    rc = lib().rf_gemm_select_config(m, n, k, ctypes.byref(cfg))
+    if rc != RF_OK:
+        raise RuntimeError("rf_gemm_select_config failed (%d): %s" % (rc, last_error()))
+    return cfg
+
+
+def variants():
+    L = lib()
+    out = []
+    for v in range(L.rf_gemm_num_variants()):
+        vals = [ctypes.c_int() for _ in range(5)]
+        L.rf_gemm_variant_info(v, *[ctypes.byref(x) for x in vals])
+        out.append(dict(variant=v, block_m=vals[0].value, block_n=vals[1].value, waves_m=vals[2].value,
+                        waves_n=vals[3].value, lds_bytes=vals[4].value))
+    return out

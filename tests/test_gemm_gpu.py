@@ -1,0 +1,197 @@
+"""GPU parity tests: the HIP path, called through the C ABI, against the CPU oracle."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cref, ref_kernel as rk
+from helpers import (ATOL, ATOL_REFERENCE, CONFIGS, RTOL, assert_close_to_oracle, assert_few_mismatches_at_reference_atol,
+                     bf16_bits, exact_problem, oracle_bf16, to_gpu)
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def rfk():
+    import radeonflow_kernels_amd as r
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    r.lib()   # raises if libgemm.so has not been built: no fallback exists
+    return r
+
+
+def _run(rfk, data, config=None, canary=0):
+    if canary:
+        g, buf = to_gpu(data, canary_elems=canary)
+    else:
+        g, buf = to_gpu(data), None
+    rfk.fp8_mm(*g, config=config)
+    torch.cuda.synchronize()
+    if buf is not None:
+        tail = buf[g[4].numel():].float().cpu().numpy()
+        assert np.all(tail == -7.0), "store past the end of C"
+    return g[4]
+
+
+GOLDEN = sorted(f for f in os.listdir(os.path.join(os.path.dirname(__file__), "golden")) if f.endswith(".npz"))
+
+
+@pytest.mark.parametrize("name", GOLDEN)
+def test_golden_fixtures(rfk, name):
+    z = np.load(os.path.join(os.path.dirname(__file__), "golden", name))
+    a = torch.from_numpy(z["a"]).view(torch.float8_e4m3fn).T
+    b = torch.from_numpy(z["b"]).view(torch.float8_e4m3fn).T
+    sa = torch.from_numpy(z["a_scale"]).T
+    sb = torch.from_numpy(z["b_scale"]).T
+    c = torch.zeros((a.shape[0], b.shape[0]), dtype=torch.bfloat16)
+    out = _run(rfk, (a, b, sa, sb, c), canary=4096)
+    assert_close_to_oracle(out, z["c_bf16"], RTOL, ATOL_REFERENCE, name)
+
+
+@pytest.mark.parametrize("gen", ["blockquant", "reference_style"])
+@pytest.mark.parametrize("m,n,k", [(256, 384, 512), (512, 576, 1024), (272, 144, 256), (16, 16, 128), (128, 7168, 256)])
+def test_every_variant_and_split(rfk, gen, m, n, k):
+    f = rk.generate_input_blockquant if gen == "blockquant" else rk.generate_input_reference_style
+    data = f(m, n, k, seed=m + n + k)
+    exp = oracle_bf16(data)
+    for v in rfk.variants():
+        for split in (1, 2, 3):
+            if split > k // 128:
+                continue
+            cfg = rfk.GemmConfig(v["variant"], split, 4)
+            out = _run(rfk, data, config=cfg, canary=1024)
+            assert_close_to_oracle(out, exp, RTOL, ATOL, "variant %r split %d" % (v, split))
+            assert_few_mismatches_at_reference_atol(out, exp, "variant %r split %d" % (v, split))
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 384, 512), (512, 576, 1024), (272, 144, 256), (16, 16, 128), (1024, 1536, 7168),
+                                   (48, 80, 7168), (33, 47, 384)])
+def test_bit_exact_on_exactly_representable_data(rfk, m, n, k):
+    """Small-integer fp8 values and power-of-two scales: every product, partial sum and fold is exact in
+    fp32 in any order, so the HIP path and the oracle must agree bit for bit. Catches any wrong index,
+    scale, K coverage or store address without being blurred by rounding."""
+    data = exact_problem(m, n, k, seed=m * 31 + n)
+    exp = oracle_bf16(data)
+    a, b, sa, sb = rk.raw_layouts(data)
+    assert np.array_equal(exp, cref.ref_gemm_blockfold(a, b, sa, sb)[1])      # exact on the CPU in both orders
+    tiled = m % 16 == 0 and n % 16 == 0
+    plans = [None]
+    if tiled:
+        plans += [rfk.GemmConfig(v["variant"], s, gm) for v in rfk.variants() for s, gm in ((1, 1), (2, 8), (3, 3))
+                  if s <= k // 128]
+    for cfg in plans:
+        out = _run(rfk, data, config=cfg, canary=1024)
+        assert np.array_equal(bf16_bits(out), exp), "plan %r" % (cfg,)
+
+
+@pytest.mark.parametrize("m,n,k", [(3, 130, 256), (1, 1, 128), (17, 64, 384), (5, 257, 128), (100, 72, 256)])
+def test_bounds_checked_kernel_on_odd_shapes(rfk, m, n, k):
+    data = rk.generate_input_reference_style(m, n, k, seed=7 * m + n)
+    cfg = rfk.select_config(m, n, k)
+    assert cfg.variant == -1
+    out = _run(rfk, data, canary=512)
+    assert_close_to_oracle(out, oracle_bf16(data), RTOL, ATOL, "checked kernel")
+    assert_few_mismatches_at_reference_atol(out, oracle_bf16(data), "checked kernel")
+
+
+# the reference's own test shapes and seeds (scripts/problems/gemm/task.yml:53-64), its input style
+REFERENCE_TESTS = [(64, 64, 128, 6635), (64, 1536, 7168, 6635), (64, 3072, 1536, 1236), (64, 576, 7168, 542),
+                   (96, 7168, 256, 1234), (96, 7168, 2048, 4153), (96, 4608, 7168, 412), (128, 7168, 2304, 624),
+                   (128, 512, 7168, 2514), (512, 4096, 512, 543), (512, 1536, 7168, 12341)]
+
+
+@pytest.mark.parametrize("m,n,k,seed", REFERENCE_TESTS)
+def test_reference_test_shapes(rfk, m, n, k, seed):
+    data = rk.generate_input_reference_style(m, n, k, seed)
+    out = _run(rfk, data, canary=1024)
+    exp = oracle_bf16(data)
+    assert_close_to_oracle(out, exp, RTOL, ATOL, "reference test shape")
+    assert_few_mismatches_at_reference_atol(out, exp, "reference test shape")
+    assert rk.check_implementation(data, out.cpu(), rtol=RTOL, atol=ATOL) == ""
+
+
+@pytest.mark.parametrize("name", ["C1", "C4", "C5"])
+def test_benchmark_configs_full_oracle(rfk, name):
+    m, n, k, seed = CONFIGS[name]
+    data = rk.generate_input_blockquant(m, n, k, seed)
+    out = _run(rfk, data, canary=1024)
+    exp = oracle_bf16(data)
+    mx = assert_close_to_oracle(out, exp, RTOL, ATOL, name)
+    bad = assert_few_mismatches_at_reference_atol(out, exp, name)
+    print("%s: max abs err %.4g, mismatches at atol 1e-3: %d of %d" % (name, mx, bad, m * n))
+
+
+@pytest.mark.parametrize("name", ["C2", "C3"])
+def test_benchmark_configs_full_size_sampled_rows_and_properties(rfk, name):
+    m, n, k, seed = CONFIGS[name]
+    data = rk.generate_input_blockquant(m, n, k, seed)
+    g = to_gpu(data)
+    rfk.fp8_mm(*g)
+    torch.cuda.synchronize()
+    base = g[4].clone()
+    # (1) sampled rows against the oracle (dequantise, fp32 accumulate over full K) and the fp64 truth
+    rng = np.random.default_rng(seed)
+    rows = np.unique(np.concatenate([[0, 1, 255, 256, m - 1], rng.integers(0, m, 43)])).astype(np.int32)
+    a, b, sa, sb = rk.raw_layouts(data)
+    _, exp16 = cref.ref_gemm_f32(a, b, sa, sb, rows=rows)
+    got = base[torch.from_numpy(rows).long().cuda()]
+    assert_close_to_oracle(got, exp16, RTOL, ATOL, name + " sampled rows")
+    assert_few_mismatches_at_reference_atol(got, exp16, name + " sampled rows")
+    truth = cref.ref_gemm_f64(a, b, sa, sb, rows=rows)
+    err = np.abs(cref.bf16_to_f32(bf16_bits(got)).astype(np.float64) - truth)
+    assert np.all(err <= 2.0 ** -8 * np.abs(truth) + ATOL), "further than one bf16 rounding + atol from the fp64 truth"
+    # (2) doubling a_scale doubles every output exactly (power of two: same roundings)
+    g2 = (g[0], g[1], (g[2].T.contiguous() * 2).T, g[3], torch.zeros_like(base))
+    rfk.fp8_mm(*g2)
+    torch.cuda.synchronize()
+    assert torch.equal(g2[4].float(), base.float() * 2)
+    # (3) permuting the rows of A (and of a_scale) permutes the rows of C bit for bit
+    perm = torch.randperm(m, generator=torch.Generator().manual_seed(seed)).cuda()
+    ap = g[0][perm].T.contiguous().T
+    sp = g[2][perm].T.contiguous().T
+    g3 = (ap, g[1], sp, g[3], torch.zeros_like(base))
+    rfk.fp8_mm(*g3)
+    torch.cuda.synchronize()
+    assert torch.equal(g3[4].view(torch.int16), base[perm].view(torch.int16))
+    # (4) zero a_scale gives an all-zero C (every element is written)
+    g4 = (g[0], g[1], torch.zeros_like(g[2].T.contiguous()).T, g[3], torch.full_like(base, 3.0))
+    rfk.fp8_mm(*g4)
+    torch.cuda.synchronize()
+    assert torch.count_nonzero(g4[4]) == 0
+
+
+def test_run_entry_writes_metrics_from_the_stream_callback(rfk):
+    from radeonflow_kernels_amd import gemm
+    data = rk.generate_input_blockquant(256, 256, 512, 3)
+    g = to_gpu(data)
+    t_ms, gflops, count = gemm.run_with_metrics(*g)
+    assert count == 0                      # the GEMM launcher leaves `count` alone
+    assert t_ms > 0 and gflops > 0
+    assert abs(gflops - 2.0 * 256 * 256 * 512 / (t_ms * 1e-3) / 1e9) <= 1e-3 * gflops
+    assert_close_to_oracle(g[4], oracle_bf16(data), RTOL, ATOL, "run()")
+
+
+def test_non_default_stream_and_repeat_calls(rfk):
+    data = rk.generate_input_reference_style(256, 512, 1024, 11)
+    exp = oracle_bf16(data)
+    g = to_gpu(data)
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        for _ in range(3):
+            g[4].zero_()
+            rfk.fp8_mm(*g)
+    s.synchronize()
+    assert_close_to_oracle(g[4], exp, RTOL, ATOL, "side stream")
+
+
+def test_status_codes(rfk):
+    L = rfk.lib()
+    t = torch.zeros(1024, dtype=torch.uint8, device="cuda")
+    p = t.data_ptr()
+    assert L.rf_fp8_gemm(p, p, p, p, p, 16, 16, 100, None) == 1      # RF_ERR_BAD_SHAPE
+    assert L.rf_fp8_gemm(p, p, p, p, p, 0, 16, 128, None) == 1
+    assert L.rf_fp8_gemm(None, p, p, p, p, 16, 16, 128, None) == 2   # RF_ERR_NULL_POINTER
+    bad = rfk.GemmConfig(99, 1, 1)
+    assert L.rf_fp8_gemm_ex(p, p, p, p, p, 16, 16, 128, ctypes.byref(bad), None) == 4
+    assert b"unsupported shape" in L.rf_gemm_last_error() or L.rf_gemm_last_error() != b""
