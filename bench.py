@@ -1,0 +1,170 @@
+#!/usr/bin/env python3
+"""Benchmark of the FP8 blockwise-scaled GEMM on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config C2] [--all] [--no-cpu]
+
+A step is one GEMM of the headline shape (M=6144, N=4608, K=7168) on synthetic inputs that are
+already resident in HBM (seeded N(0,1) fp32, quantised to e4m3fn with amax/448 block scales).
+Prints ONE JSON line on stdout; per-config tables (with --all) go to stderr.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP8_TFLOPS = 5000.0      # MI355X published dense fp8 MFMA peak
+PEAK_HBM_GBS = 8000.0         # MI355X published HBM3E bandwidth
+
+CONFIGS = {
+    "C1": (1024, 1536, 7168, 8135),
+    "C2": (6144, 4608, 7168, 65436),
+    "C3": (6144, 7168, 2048, 76547),
+    "C4": (6144, 7168, 256, 764243),
+    "C5": (1024, 576, 7168, 12346),
+}
+RTOL, ATOL, ATOL_REFERENCE = 2e-2, 1e-2, 1e-3
+
+
+def algorithmic_bytes(m, n, k):
+    qk, qn = k // 128, (n + 127) // 128
+    return m * k + n * k + 2 * m * n + 4 * m * qk + 4 * qn * qk
+
+
+def to_gpu(data):
+    a, b, sa, sb, c = data
+
+    def colmajor(t):
+        return t.T.contiguous().cuda().T
+    return colmajor(a), colmajor(b), colmajor(sa), colmajor(sb), torch.zeros(c.shape, dtype=torch.bfloat16, device="cuda")
+
+
+def time_gemm(rfk, g, steps, warmup, stream):
+    """Average microseconds per GEMM over `steps` back-to-back launches, HIP events on the launch stream."""
+    with torch.cuda.stream(stream):
+        for _ in range(warmup):
+            rfk.fp8_mm(*g)
+        stream.synchronize()
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(steps):
+            rfk.fp8_mm(*g)
+        e1.record(stream)
+        stream.synchronize()
+        torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / steps
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--config", default="C2", choices=sorted(CONFIGS))
+    ap.add_argument("--all", action="store_true", help="also time the other four configurations (stderr table)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity gate")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus %d is not supported (the path shards over M or N "
+              "without any exchange, see DESIGN.md)" % args.gpus, file=sys.stderr)
+        return 2
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+
+    import radeonflow_kernels_amd as rfk
+    rfk.lib()        # fails loudly if libgemm.so is missing
+    from oracle import cref, ref_kernel as rk      # checker + CPU baseline only
+
+    prop = torch.cuda.get_device_properties(0)
+    clock_mhz = getattr(prop, "clock_rate", 2400000) / 1e3
+    derived_peak = prop.multi_processor_count * clock_mhz * 1e6 * 8192 / 1e12
+    stream = torch.cuda.Stream()
+
+    m, n, k, seed = CONFIGS[args.config]
+    t0 = time.time()
+    data = rk.generate_input_blockquant(m, n, k, seed)
+    g = to_gpu(data)
+    gen_s = time.time() - t0
+
+    us = time_gemm(rfk, g, args.steps, args.warmup, stream)
+    flop = 2.0 * m * n * k
+    tflops = flop / us / 1e6
+    gbs = algorithmic_bytes(m, n, k) / us / 1e3
+    cfg = rfk.select_config(m, n, k)
+    mfma_bound = flop / (PEAK_FP8_TFLOPS * 1e12) >= algorithmic_bytes(m, n, k) / (PEAK_HBM_GBS * 1e9)
+    if mfma_bound:
+        roofline = {"bound": "mfma", "achieved": round(tflops, 2), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(tflops / PEAK_FP8_TFLOPS, 4), "traffic": None}
+    else:
+        roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}
+    roofline["kernel"] = "gemm_fp8_blockscale_tile (variant %d, split_k %d)" % (cfg.variant, cfg.split_k)
+    roofline["avg_launch_us"] = round(us, 2)
+    roofline["algorithmic_flop_per_launch"] = flop
+    roofline["algorithmic_bytes_per_launch"] = algorithmic_bytes(m, n, k)
+
+    out = {
+        "metric": "TFLOP/s per blockscaled fp8 GEMM (M=%d,N=%d,K=%d)" % (m, n, k),
+        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(us / 1e3, 5), "us_per_gemm": round(us, 2),
+        "pct_fp8_mfma_peak": round(100 * tflops / PEAK_FP8_TFLOPS, 2),
+        "achieved_hbm_gbs_algorithmic": round(gbs, 1),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3fn",
+        "data": "synthetic (seeded N(0,1) fp32 -> e4m3fn, amax/448 block scales), random inputs resident in HBM",
+        "config": {"workload": "%s: blockscaled fp8 GEMM M=%d N=%d K=%d, a[K][M] b[K][N] fp8, fp32 scales, bf16 C"
+                               % (args.config, m, n, k),
+                   "plan": {"variant": cfg.variant, "split_k": cfg.split_k, "group_m": cfg.group_m},
+                   "device": prop.name, "compute_units": prop.multi_processor_count, "clock_mhz": clock_mhz,
+                   "derived_fp8_peak_tflops": round(derived_peak, 1), "input_generation_s": round(gen_s, 2)},
+        "roofline": roofline,
+    }
+
+    if not args.no_cpu:
+        # CPU baseline = the oracle's torch restatement of the reference path (dequantise, fp32 matmul, bf16)
+        # on the host cores, whole workload, one timed run after a small warm-up. Also the parity gate.
+        a, b, sa, sb, c = data
+        warm = (a[:128], b, sa[:128], sb, torch.zeros((128, n), dtype=torch.bfloat16))
+        rk.ref_kernel(warm)
+        t0 = time.perf_counter()
+        expect = rk.ref_kernel((a, b, sa, sb, torch.zeros((m, n), dtype=torch.bfloat16)))
+        cpu_s = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": round(flop / cpu_s / 1e12, 4), "unit": "TFLOP/s",
+                               "cores": torch.get_num_threads(), "kind": "port", "seconds": round(cpu_s, 2),
+                               "host_cpu_count": os.cpu_count(),
+                               "sample": "whole %s workload once (dequantise + fp32 matmul + bf16 cast), torch CPU" % args.config}
+        with torch.cuda.stream(stream):
+            g[4].zero_()
+            rfk.fp8_mm(*g)
+            stream.synchronize()
+        got = g[4].cpu().view(torch.uint16).numpy()
+        exp = expect.view(torch.uint16).numpy()
+        bad, mx, _ = cref.allclose(got, exp, RTOL, ATOL)
+        bad_ref, _, _ = cref.allclose(got, exp, RTOL, ATOL_REFERENCE)
+        out["parity"] = {"rtol": RTOL, "atol": ATOL, "mismatches": bad, "max_abs_err": round(mx, 5),
+                         "mismatches_at_reference_atol_1e-3": bad_ref, "elements": int(m * n), "pass": bad == 0}
+
+    if args.all:
+        print("%-3s %-20s %10s %10s %8s %10s  %s" % ("cfg", "shape", "us", "TFLOP/s", "%peak", "GB/s(alg)", "plan"), file=sys.stderr)
+        for name, (mm, nn, kk, sd) in CONFIGS.items():
+            gg = to_gpu(rk.generate_input_blockquant(mm, nn, kk, sd))
+            u = time_gemm(rfk, gg, args.steps, args.warmup, stream)
+            tf = 2.0 * mm * nn * kk / u / 1e6
+            print("%-3s %-20s %10.2f %10.1f %8.2f %10.1f  %r" % (name, "%dx%dx%d" % (mm, nn, kk), u, tf,
+                  100 * tf / PEAK_FP8_TFLOPS, algorithmic_bytes(mm, nn, kk) / u / 1e3, rfk.select_config(mm, nn, kk)),
+                  file=sys.stderr)
+            del gg
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
