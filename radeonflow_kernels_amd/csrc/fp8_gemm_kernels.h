@@ -89,10 +89,14 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
     constexpr int NW = WAVES_M * WAVES_N;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     constexpr int TM = WM / 16, TN = WN / 16;
-    constexpr int STAGE_A = BK * BM, STAGE_B = BK * BN, STAGE = STAGE_A + STAGE_B;
+    // one LDS stage: A[128][BM] bytes, B[128][BN] bytes, then BM fp32 a_scale values
+    constexpr int STAGE_A = BK * BM, STAGE_B = BK * BN, STAGE_S = BM * 4, STAGE = STAGE_A + STAGE_B + STAGE_S;
     constexpr int INST_A = STAGE_A / 1024 / NW, INST_B = STAGE_B / 1024 / NW;   // 1 KiB per wave instruction
+    constexpr int NSC = BM / 64;                                                // scale loads: 64 floats each
     static_assert(STAGE_A % (1024 * NW) == 0 && STAGE_B % (1024 * NW) == 0, "loads must divide evenly over waves");
+    static_assert(NSC <= NW, "one scale load per wave at most");
     static_assert(WN <= 128 && 128 % WN == 0, "a wave's N range must sit inside one scale block");
+    static_assert(TM % 4 == 0, "scales are read back four at a time");
     constexpr int CPR_A = BM / 16, CPR_B = BN / 16;          // 16-byte chunks per LDS row
     constexpr int RPI_A = 1024 / BM, RPI_B = 1024 / BN;      // rows per load instruction
 
@@ -112,7 +116,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
     const int kb_end = kb_begin + kb_per_split < QK ? kb_begin + kb_per_split : QK;
 
     // ---- global -> LDS: per-lane source offsets inside one K block (rows k_local, swizzled chunk) ----
-    uint32_t goff_a[INST_A], goff_b[INST_B];
+    uint32_t goff_a[INST_A], goff_b[INST_B], goff_s;
 #pragma unroll
     for (int i = 0; i < INST_A; i++) {
         int q = wave * INST_A + i;
@@ -131,19 +135,42 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
         if (n + 16 > N) n = N - 16;
         goff_b[i] = (uint32_t)kl * (uint32_t)N + (uint32_t)n;
     }
-    auto issue_stage = [&](int stage, int kb) {
-        const uint8_t *ak = A + (size_t)kb * BK * M;
-        const uint8_t *bk = B + (size_t)kb * BK * N;
-        uint8_t *sa_lds = lds + stage * STAGE;
-        uint8_t *sb_lds = sa_lds + STAGE_A;
-#pragma unroll
-        for (int i = 0; i < INST_A; i++)
-            __builtin_amdgcn_global_load_lds((const RF_GLOBAL void *)(ak + goff_a[i]),
-                                             (RF_LDS void *)(sa_lds + (wave * INST_A + i) * 1024), 16, 0, 0);
-#pragma unroll
-        for (int i = 0; i < INST_B; i++)
-            __builtin_amdgcn_global_load_lds((const RF_GLOBAL void *)(bk + goff_b[i]),
-                                             (RF_LDS void *)(sb_lds + (wave * INST_B + i) * 1024), 16, 0, 0);
+    {
+        // a_scale slot s of the stage holds the scale of row (s/WM)*WM + 16*(s%TM) + (s%WM)/TM of the tile, so that
+        // the TM scales a lane needs (its column L of every m-tile of its wave) are contiguous in LDS.
+        int sl = (wave < NSC ? wave : 0) * 64 + lane;
+        int r = sl % WM;
+        int m = m0 + (sl / WM) * WM + 16 * (r % TM) + r / TM;
+        if (m > M - 1) m = M - 1;
+        goff_s = (uint32_t)m * 4u;
+    }
+    // The LDS-DMA loads are issued through inline asm on purpose: the compiler cannot tell which stage a
+    // transpose read touches, so for builtin LDS-DMA loads it waits for vmcnt(0) before the first LDS read
+    // that follows them, which serialises the prefetch with the compute it is meant to overlap. Here the
+    // kernel owns the wait: one s_waitcnt vmcnt(0) before the barrier at the top of the next iteration.
+    // Addressing: 64-bit SGPR base (advances by 128 rows per K block) + per-lane 32-bit offset; M0 holds
+    // the LDS destination of the instruction (lane l lands at M0 + 16*l, or M0 + 4*l for the dword form).
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(RF_LDS uint8_t *)lds;
+    constexpr int NDMA = INST_A + INST_B + 1;
+    // DMA instruction `d` of this wave for K block kb into `stage`: A rows, then B rows, then the scales
+    auto issue_dma = [&](int d, int stage, int kb) {
+        if (d < INST_A) {
+            const uint8_t *ak = A + (size_t)kb * BK * M;
+            const uint32_t dst = lds_base + stage * STAGE + (wave * INST_A + d) * 1024;
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                         :: "v"(goff_a[d < INST_A ? d : 0]), "s"(ak), "s"(dst) : "memory");
+        } else if (d < INST_A + INST_B) {
+            const int e = d - INST_A;
+            const uint8_t *bk = B + (size_t)kb * BK * N;
+            const uint32_t dst = lds_base + stage * STAGE + STAGE_A + (wave * INST_B + e) * 1024;
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                         :: "v"(goff_b[e >= 0 && e < INST_B ? e : 0]), "s"(bk), "s"(dst) : "memory");
+        } else if (wave < NSC) {
+            const float *sk = SA + (size_t)kb * M;
+            const uint32_t dst = lds_base + stage * STAGE + STAGE_A + STAGE_B + wave * 256;
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+                         :: "v"(goff_s), "s"(sk), "s"(dst) : "memory");
+        }
     };
 
     // ---- LDS -> MFMA operands: per-lane byte offsets of the transpose reads (stage 0, t = 0) ----
@@ -162,14 +189,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
         for (int i = 0; i < TN; i++)
             boff[i] = STAGE_A + krow * BN + (((wn * TN + i) ^ sw) << 4) + 8 * (L & 1);
     }
+    const uint32_t soff = STAGE_A + STAGE_B + (wm * WM + L * TM) * 4;   // this lane's TM scales
 
-    // ---- scales: lane needs a_scale[kb][m] for its column m of every m-tile, and one b_scale ----
-    int srow[TM];
-#pragma unroll
-    for (int j = 0; j < TM; j++) {
-        int m = m0 + wm * WM + 16 * j + L;
-        srow[j] = m < M ? m : M - 1;
-    }
     int nb = (n0 + wn * WN) >> 7;
     if (nb > QN - 1) nb = QN - 1;
 
@@ -179,58 +200,86 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
 #pragma unroll
         for (int i = 0; i < TN; i++) acc[j][i] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-    float sa_next[TM], sb_next;
-    auto load_scales = [&](int kb) {
-#pragma unroll
-        for (int j = 0; j < TM; j++) sa_next[j] = SA[(size_t)kb * M + srow[j]];
-        sb_next = SB[(size_t)kb * QN + nb];
-    };
+    // b_scale is wave-uniform, but it is fetched with a vector load on purpose: a scalar load returns out of
+    // order with LDS reads on the same counter and would force every LDS wait in the loop down to zero.
+    int vzero;
+    asm volatile("v_mov_b32 %0, 0" : "=v"(vzero));
+    float sb_next = 0.f;
 
     if (kb_begin < kb_end) {
-        issue_stage(0, kb_begin);
-        load_scales(kb_begin);
+#pragma unroll
+        for (int d = 0; d < NDMA; d++) issue_dma(d, 0, kb_begin);
+        sb_next = SB[(size_t)kb_begin * QN + nb + vzero];
     }
+    // One K block per iteration, software-pipelined by hand. MFMA t = (m-tile j, n-tile i) in row-major order:
+    //   * its partial sum goes to a ring of PR register tiles and is folded into the accumulator LAG MFMAs
+    //     later, so the VALU folds run while later MFMAs occupy the matrix pipe;
+    //   * the A-matrix fragment of m-tile j+1 is fetched from LDS while the MFMAs of m-tile j issue;
+    //   * the LDS-DMA loads of the next K block are dealt out one per MFMA slot, so that no wave sits behind a
+    //     burst of vector-memory instructions at the start of the iteration.
+    // sched_barrier(0) after every slot pins this order; the compiler still places the waitcnts and hazard nops.
+    constexpr int PR = 4, LAG = 3, NMFMA = TM * TN;
+    static_assert(NDMA <= NMFMA, "one DMA instruction per MFMA slot");
     for (int kb = kb_begin, it = 0; kb < kb_end; ++kb, ++it) {
         // my loads for this stage have landed; after the barrier everyone's have, and everyone has
         // finished reading the other stage (computed in the previous iteration)
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        float s[TM];
-#pragma unroll
-        for (int j = 0; j < TM; j++) s[j] = sa_next[j] * sb_next;
-        if (kb + 1 < kb_end) {
-            issue_stage((it + 1) & 1, kb + 1);
-            load_scales(kb + 1);
-        }
+        const float sb_cur = sb_next;
+        // the last iteration re-fetches its own block: harmless, and it keeps the loop body free of branches
+        const int kn = kb + 1 < kb_end ? kb + 1 : kb;
+        const int nstage = (it + 1) & 1;
+        sb_next = SB[(size_t)kn * QN + nb + vzero];
         const uint32_t sbase = (it & 1) * STAGE;
-        i32x8 bfrag[TN];
+        i32x8 bfrag[TN], afrag[2];
+        f32x4 pring[PR];
+        float s[TM];
+        auto rd = [&](uint32_t off) {
+            return __builtin_amdgcn_ds_read_tr8_b64_v2i32((RF_LDS i32x2 *)(lds + sbase + off));
+        };
+        // first operands: n-tile 0 and m-tile 0, then the scales and the other n-tiles
 #pragma unroll
-        for (int i = 0; i < TN; i++) {
+        for (int t = 0; t < 4; t++) { i32x2 v = rd(boff[0] + t * 8 * BN); bfrag[0][2 * t] = v[0]; bfrag[0][2 * t + 1] = v[1]; }
 #pragma unroll
-            for (int t = 0; t < 4; t++) {
-                i32x2 v = __builtin_amdgcn_ds_read_tr8_b64_v2i32((RF_LDS i32x2 *)(lds + sbase + boff[i] + t * 8 * BN));
-                bfrag[i][2 * t] = v[0];
-                bfrag[i][2 * t + 1] = v[1];
-            }
+        for (int t = 0; t < 4; t++) { i32x2 v = rd(aoff[0] + t * 8 * BM); afrag[0][2 * t] = v[0]; afrag[0][2 * t + 1] = v[1]; }
+#pragma unroll
+        for (int q = 0; q < TM / 4; q++) {
+            f32x4 v = *(RF_LDS f32x4 *)(lds + sbase + soff + q * 16);
+#pragma unroll
+            for (int e = 0; e < 4; e++) s[4 * q + e] = v[e] * sb_cur;
         }
 #pragma unroll
-        for (int j = 0; j < TM; j++) {
-            i32x8 afrag;
+        for (int i = 1; i < TN; i++)
 #pragma unroll
-            for (int t = 0; t < 4; t++) {
-                i32x2 v = __builtin_amdgcn_ds_read_tr8_b64_v2i32((RF_LDS i32x2 *)(lds + sbase + aoff[j] + t * 8 * BM));
-                afrag[2 * t] = v[0];
-                afrag[2 * t + 1] = v[1];
+            for (int t = 0; t < 4; t++) { i32x2 v = rd(boff[i] + t * 8 * BN); bfrag[i][2 * t] = v[0]; bfrag[i][2 * t + 1] = v[1]; }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < NMFMA + LAG; t++) {
+            if (t < NMFMA) {
+                const int j = t / TN, i = t % TN;
+                pring[t % PR] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                    bfrag[i], afrag[j & 1], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                if (t < NDMA) issue_dma(t, nstage, kn);
+                if (j + 1 < TM && i == 0) {   // the next m-tile's fragment, a whole m-tile ahead of its use
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        i32x2 v = rd(aoff[j + 1] + q * 8 * BM);
+                        afrag[(j + 1) & 1][2 * q] = v[0];
+                        afrag[(j + 1) & 1][2 * q + 1] = v[1];
+                    }
+                }
             }
+            if (t >= LAG) {
+                const int u = t - LAG, j = u / TN, i = u % TN;
 #pragma unroll
-            for (int i = 0; i < TN; i++) {
-                f32x4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bfrag[i], afrag, (f32x4){0.f, 0.f, 0.f, 0.f},
-                                                                          0, 0, 0, 0, 0, 0);
-#pragma unroll
-                for (int e = 0; e < 4; e++) acc[j][i][e] = __builtin_fmaf(s[j], p[e], acc[j][i][e]);
+                for (int e = 0; e < 4; e++) acc[j][i][e] = __builtin_fmaf(s[j], pring[u % PR][e], acc[j][i][e]);
             }
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
+    // LDS-DMA writes of the last (redundant) prefetch must land before this workgroup's LDS can be handed on
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
     // ---- epilogue: lane holds C[m][n..n+3] per tile ----
 #pragma unroll

@@ -37,7 +37,7 @@ typedef void (*tile_kernel_t)(const uint8_t *, const uint8_t *, const float *, c
 struct Variant {
     int bm, bn, waves_m, waves_n;
     tile_kernel_t direct, partial;
-    int lds_bytes() const { return 2 * rf::BK * (bm + bn); }
+    int lds_bytes() const { return 2 * (rf::BK * (bm + bn) + 4 * bm); }
     int threads() const { return waves_m * waves_n * 64; }
 };
 #define RF_VARIANT(BM, BN, WM, WN)                                                         \
