@@ -116,24 +116,36 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
     const int kb_end = kb_begin + kb_per_split < QK ? kb_begin + kb_per_split : QK;
 
     // ---- global -> LDS: per-lane source offsets inside one K block (rows k_local, swizzled chunk) ----
-    uint32_t goff_a[INST_A], goff_b[INST_B], goff_s;
+    // Load instruction i of this wave covers rows (wave*INST + i)*RPI .. +RPI-1. Its per-lane offset differs from
+    // that of another instruction only by a wave-uniform amount when both see the same row swizzle, i.e. the same
+    // (k & 7) and (k >> 5) & 1 for every lane. So only one VGPR per swizzle class is kept; the rest is scalar.
+    constexpr int PER_A = (8 / RPI_A) > 0 ? (8 / RPI_A) : 1, PER_B = (8 / RPI_B) > 0 ? (8 / RPI_B) : 1;
+    constexpr int GRP_A = (INST_A * RPI_A + 31) / 32, GRP_B = (INST_B * RPI_B + 31) / 32;   // 32-row groups per wave
+    constexpr int NCLS_A = (PER_A < INST_A ? PER_A : INST_A) * GRP_A, NCLS_B = (PER_B < INST_B ? PER_B : INST_B) * GRP_B;
+    static_assert((INST_A * RPI_A) % 32 == 0 || INST_A * RPI_A < 32, "a wave's rows cover whole 32-row groups");
+    static_assert((INST_B * RPI_B) % 32 == 0 || INST_B * RPI_B < 32, "a wave's rows cover whole 32-row groups");
+    auto cls_a = [](int i) { return i % PER_A + PER_A * (i * RPI_A / 32); };   // class of instruction i
+    auto rep_a = [](int c) { return c % PER_A + (c / PER_A) * (32 / RPI_A); }; // first instruction of class c
+    auto cls_b = [](int i) { return i % PER_B + PER_B * (i * RPI_B / 32); };
+    auto rep_b = [](int c) { return c % PER_B + (c / PER_B) * (32 / RPI_B); };
+    uint32_t goff_a[NCLS_A], goff_b[NCLS_B], goff_s;
 #pragma unroll
-    for (int i = 0; i < INST_A; i++) {
-        int q = wave * INST_A + i;
+    for (int c_ = 0; c_ < NCLS_A; c_++) {
+        int q = wave * INST_A + rep_a(c_);
         int kl = q * RPI_A + lane / CPR_A;
         int c = (lane % CPR_A) ^ swizzle_of_row<BM>(kl);
         int m = m0 + c * 16;
         if (m + 16 > M) m = M - 16;                           // rows past M: any valid bytes will do
-        goff_a[i] = (uint32_t)kl * (uint32_t)M + (uint32_t)m;
+        goff_a[c_] = (uint32_t)(lane / CPR_A) * (uint32_t)M + (uint32_t)m;
     }
 #pragma unroll
-    for (int i = 0; i < INST_B; i++) {
-        int q = wave * INST_B + i;
+    for (int c_ = 0; c_ < NCLS_B; c_++) {
+        int q = wave * INST_B + rep_b(c_);
         int kl = q * RPI_B + lane / CPR_B;
         int c = (lane % CPR_B) ^ swizzle_of_row<BN>(kl);
         int n = n0 + c * 16;
         if (n + 16 > N) n = N - 16;
-        goff_b[i] = (uint32_t)kl * (uint32_t)N + (uint32_t)n;
+        goff_b[c_] = (uint32_t)(lane / CPR_B) * (uint32_t)N + (uint32_t)n;
     }
     {
         // a_scale slot s of the stage holds the scale of row (s/WM)*WM + 16*(s%TM) + (s%WM)/TM of the tile, so that
@@ -155,16 +167,16 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
     // DMA instruction `d` of this wave for K block kb into `stage`: A rows, then B rows, then the scales
     auto issue_dma = [&](int d, int stage, int kb) {
         if (d < INST_A) {
-            const uint8_t *ak = A + (size_t)kb * BK * M;
+            const uint8_t *ak = A + ((size_t)kb * BK + (size_t)(wave * INST_A + d) * RPI_A) * M;
             const uint32_t dst = lds_base + stage * STAGE + (wave * INST_A + d) * 1024;
             asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                         :: "v"(goff_a[d < INST_A ? d : 0]), "s"(ak), "s"(dst) : "memory");
+                         :: "v"(goff_a[cls_a(d < INST_A ? d : 0)]), "s"(ak), "s"(dst) : "memory");
         } else if (d < INST_A + INST_B) {
-            const int e = d - INST_A;
-            const uint8_t *bk = B + (size_t)kb * BK * N;
+            const int e = d - INST_A < INST_B ? d - INST_A : 0;
+            const uint8_t *bk = B + ((size_t)kb * BK + (size_t)(wave * INST_B + e) * RPI_B) * N;
             const uint32_t dst = lds_base + stage * STAGE + STAGE_A + (wave * INST_B + e) * 1024;
             asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                         :: "v"(goff_b[e >= 0 && e < INST_B ? e : 0]), "s"(bk), "s"(dst) : "memory");
+                         :: "v"(goff_b[cls_b(e >= 0 ? e : 0)]), "s"(bk), "s"(dst) : "memory");
         } else if (wave < NSC) {
             const float *sk = SA + (size_t)kb * M;
             const uint32_t dst = lds_base + stage * STAGE + STAGE_A + STAGE_B + wave * 256;
@@ -176,19 +188,11 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
     // ---- LDS -> MFMA operands: per-lane byte offsets of the transpose reads (stage 0, t = 0) ----
     // lane (L,g) of read t points at row k = 32g + 8t + L/2, half (L&1) of 16-byte chunk c.
     const int krow = 32 * g + (L >> 1);
-    uint32_t aoff[TM], boff[TN];
-    {
-        const int sw = swizzle_of_row<BM>(krow);              // independent of t (8t leaves k&7 and k>>5 alone)
-#pragma unroll
-        for (int j = 0; j < TM; j++)
-            aoff[j] = krow * BM + (((wm * TM + j) ^ sw) << 4) + 8 * (L & 1);
-    }
-    {
-        const int sw = swizzle_of_row<BN>(krow);
-#pragma unroll
-        for (int i = 0; i < TN; i++)
-            boff[i] = STAGE_A + krow * BN + (((wn * TN + i) ^ sw) << 4) + 8 * (L & 1);
-    }
+    // chunk index of m-tile j is (wm*TM + j) ^ sw = ((wm*TM) ^ sw) ^ j because j < TM and wm*TM is a multiple of TM
+    // (TM, TN powers of two): one base register per operand, the tile index is XORed in at the use.
+    static_assert((TM & (TM - 1)) == 0 && (TN & (TN - 1)) == 0, "tile counts are powers of two");
+    const uint32_t aoff_base = krow * BM + (((wm * TM) ^ swizzle_of_row<BM>(krow)) << 4) + 8 * (L & 1);
+    const uint32_t boff_base = krow * BN + (((wn * TN) ^ swizzle_of_row<BN>(krow)) << 4) + 8 * (L & 1);
     const uint32_t soff = STAGE_A + STAGE_B + (wm * WM + L * TM) * 4;   // this lane's TM scales
 
     int nb = (n0 + wn * WN) >> 7;
@@ -239,9 +243,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
         };
         // first operands: n-tile 0 and m-tile 0, then the scales and the other n-tiles
 #pragma unroll
-        for (int t = 0; t < 4; t++) { i32x2 v = rd(boff[0] + t * 8 * BN); bfrag[0][2 * t] = v[0]; bfrag[0][2 * t + 1] = v[1]; }
+        for (int t = 0; t < 4; t++) { i32x2 v = rd((boff_base ^ (0 << 4)) + STAGE_A + t * 8 * BN); bfrag[0][2 * t] = v[0]; bfrag[0][2 * t + 1] = v[1]; }
 #pragma unroll
-        for (int t = 0; t < 4; t++) { i32x2 v = rd(aoff[0] + t * 8 * BM); afrag[0][2 * t] = v[0]; afrag[0][2 * t + 1] = v[1]; }
+        for (int t = 0; t < 4; t++) { i32x2 v = rd((aoff_base ^ (0 << 4)) + t * 8 * BM); afrag[0][2 * t] = v[0]; afrag[0][2 * t + 1] = v[1]; }
 #pragma unroll
         for (int q = 0; q < TM / 4; q++) {
             f32x4 v = *(RF_LDS f32x4 *)(lds + sbase + soff + q * 16);
@@ -251,7 +255,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
 #pragma unroll
         for (int i = 1; i < TN; i++)
 #pragma unroll
-            for (int t = 0; t < 4; t++) { i32x2 v = rd(boff[i] + t * 8 * BN); bfrag[i][2 * t] = v[0]; bfrag[i][2 * t + 1] = v[1]; }
+            for (int t = 0; t < 4; t++) { i32x2 v = rd((boff_base ^ (i << 4)) + STAGE_A + t * 8 * BN); bfrag[i][2 * t] = v[0]; bfrag[i][2 * t + 1] = v[1]; }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int t = 0; t < NMFMA + LAG; t++) {
@@ -264,7 +268,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
                 if (j + 1 < TM && i == 0) {   // the next m-tile's fragment, a whole m-tile ahead of its use
 #pragma unroll
                     for (int q = 0; q < 4; q++) {
-                        i32x2 v = rd(aoff[j + 1] + q * 8 * BM);
+                        i32x2 v = rd((aoff_base ^ ((j + 1) << 4)) + q * 8 * BM);
                         afrag[(j + 1) & 1][2 * q] = v[0];
                         afrag[(j + 1) & 1][2 * q + 1] = v[1];
                     }
