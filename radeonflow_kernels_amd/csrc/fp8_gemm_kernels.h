@@ -263,6 +263,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
                 const int j = t / TN, i = t % TN;
                 pring[t % PR] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
                     bfrag[i], afrag[j & 1], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+                asm volatile("" : "+v"(pring[t % PR]));      // anchor: the MFMA is issued here, not later
                 __builtin_amdgcn_sched_barrier(0);
                 if (t < NDMA) issue_dma(t, nstage, kn);
                 if (j + 1 < TM && i == 0) {   // the next m-tile's fragment, a whole m-tile ahead of its use
@@ -278,6 +279,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
                 const int u = t - LAG, j = u / TN, i = u % TN;
 #pragma unroll
                 for (int e = 0; e < 4; e++) acc[j][i][e] = __builtin_fmaf(s[j], pring[u % PR][e], acc[j][i][e]);
+                asm volatile("" : "+v"(acc[j][i]));          // anchor: the fold happens in this slot
             }
             __builtin_amdgcn_sched_barrier(0);
         }
