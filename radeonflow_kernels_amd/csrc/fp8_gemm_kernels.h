@@ -208,83 +208,142 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
     // order with LDS reads on the same counter and would force every LDS wait in the loop down to zero.
     int vzero;
     asm volatile("v_mov_b32 %0, 0" : "=v"(vzero));
-    float sb_next = 0.f;
-
-    if (kb_begin < kb_end) {
-#pragma unroll
-        for (int d = 0; d < NDMA; d++) issue_dma(d, 0, kb_begin);
-        sb_next = SB[(size_t)kb_begin * QN + nb + vzero];
-    }
-    // One K block per iteration, software-pipelined by hand. MFMA t = (m-tile j, n-tile i) in row-major order:
-    //   * its partial sum goes to a ring of PR register tiles and is folded into the accumulator LAG MFMAs
-    //     later, so the VALU folds run while later MFMAs occupy the matrix pipe;
+    // ---- main loop: one K block per iteration, software-pipelined by hand across iterations ----
+    // MFMA slot t = (m-tile j, n-tile i), row-major. In steady state the matrix pipe never waits for a K-block
+    // boundary:
+    //   * the partial sum of slot t goes to a ring of PR register tiles and is folded into the accumulator LAG
+    //     slots later (the last LAG folds of a K block run in the first slots of the next one);
     //   * the A-matrix fragment of m-tile j+1 is fetched from LDS while the MFMAs of m-tile j issue;
-    //   * the LDS-DMA loads of the next K block are dealt out one per MFMA slot, so that no wave sits behind a
-    //     burst of vector-memory instructions at the start of the iteration.
-    // sched_barrier(0) after every slot pins this order; the compiler still places the waitcnts and hazard nops.
-    constexpr int PR = 4, LAG = 3, NMFMA = TM * TN;
-    static_assert(NDMA <= NMFMA, "one DMA instruction per MFMA slot");
-    for (int kb = kb_begin, it = 0; kb < kb_end; ++kb, ++it) {
-        // my loads for this stage have landed; after the barrier everyone's have, and everyone has
-        // finished reading the other stage (computed in the previous iteration)
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        const float sb_cur = sb_next;
-        // the last iteration re-fetches its own block: harmless, and it keeps the loop body free of branches
-        const int kn = kb + 1 < kb_end ? kb + 1 : kb;
-        const int nstage = (it + 1) & 1;
-        sb_next = SB[(size_t)kn * QN + nb + vzero];
-        const uint32_t sbase = (it & 1) * STAGE;
-        i32x8 bfrag[TN], afrag[2];
-        f32x4 pring[PR];
-        float s[TM];
-        auto rd = [&](uint32_t off) {
-            return __builtin_amdgcn_ds_read_tr8_b64_v2i32((RF_LDS i32x2 *)(lds + sbase + off));
-        };
-        // first operands: n-tile 0 and m-tile 0, then the scales and the other n-tiles
+    //   * the barrier that publishes the next stage sits before the LAST m-tile's slots (slot BAR_SLOT). In those
+    //     slots each B-matrix fragment is dead as soon as its MFMA has issued and is refilled from the next
+    //     stage, together with the first A fragment and the scales of the next K block;
+    //   * after that barrier the stage just consumed is free: the LDS-DMA loads of K block kb+2 start there, one
+    //     per slot, and run on into the first slots of the next iteration.
+    // An empty volatile asm after each MFMA / fold anchors it in its slot, sched_barrier(0) keeps the slots apart;
+    // the compiler still places the waitcnts and hazard nops.
+    constexpr int PR = 4, LAG = 3, NMFMA = TM * TN, BAR_SLOT = (TM - 1) * TN;
+    static_assert(LAG < TN && LAG < PR, "lagged folds of a K block stay inside its last m-tile row");
+    static_assert(TM % 2 == 0, "the last m-tile uses afrag[1], so afrag[0] is free for the next block");
+    static_assert(NDMA - TN <= BAR_SLOT, "the DMA batch finishes well before the barrier that needs it");
+    const int kb_last = kb_end - 1;
+    auto clamp_kb = [&](int kb) { return kb < kb_last ? kb : kb_last; };   // past the end: re-fetch the last block
+
+    i32x8 bfrag[TN], afrag[2];
+    f32x4 pring[PR];
+    float s[TM], sraw[TM], sb_cur = 0.f, sb_next = 0.f;
 #pragma unroll
-        for (int t = 0; t < 4; t++) { i32x2 v = rd((boff_base ^ (0 << 4)) + STAGE_A + t * 8 * BN); bfrag[0][2 * t] = v[0]; bfrag[0][2 * t + 1] = v[1]; }
+    for (int r = 0; r < PR; r++) pring[r] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int t = 0; t < 4; t++) { i32x2 v = rd((aoff_base ^ (0 << 4)) + t * 8 * BM); afrag[0][2 * t] = v[0]; afrag[0][2 * t + 1] = v[1]; }
+    for (int j = 0; j < TM; j++) s[j] = 0.f;
+
+    auto rd = [&](uint32_t stage_base, uint32_t off) {
+        return __builtin_amdgcn_ds_read_tr8_b64_v2i32((RF_LDS i32x2 *)(lds + stage_base + off));
+    };
+    auto read_bfrag = [&](int i, uint32_t stage_base) {
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            i32x2 v = rd(stage_base, (boff_base ^ (i << 4)) + STAGE_A + t * 8 * BN);
+            bfrag[i][2 * t] = v[0];
+            bfrag[i][2 * t + 1] = v[1];
+        }
+    };
+    auto read_afrag = [&](int buf, int j, uint32_t stage_base) {
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            i32x2 v = rd(stage_base, (aoff_base ^ (j << 4)) + t * 8 * BM);
+            afrag[buf][2 * t] = v[0];
+            afrag[buf][2 * t + 1] = v[1];
+        }
+    };
+    auto read_scales = [&](uint32_t stage_base) {
 #pragma unroll
         for (int q = 0; q < TM / 4; q++) {
-            f32x4 v = *(RF_LDS f32x4 *)(lds + sbase + soff + q * 16);
+            f32x4 v = *(RF_LDS f32x4 *)(lds + stage_base + soff + q * 16);
 #pragma unroll
-            for (int e = 0; e < 4; e++) s[4 * q + e] = v[e] * sb_cur;
+            for (int e = 0; e < 4; e++) sraw[4 * q + e] = v[e];
         }
+    };
+
+    if (kb_begin < kb_end) {
+        // prologue: stage 0 <- first K block, then its first operands; stage 1 <- second K block
 #pragma unroll
-        for (int i = 1; i < TN; i++)
+        for (int d = 0; d < NDMA; d++) issue_dma(d, 0, kb_begin);
+        sb_cur = SB[(size_t)kb_begin * QN + nb + vzero];
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        asm volatile("" : "+v"(sb_cur));
+        __syncthreads();
+        read_bfrag(0, 0);
+        read_afrag(0, 0, 0);
+        read_scales(0);
 #pragma unroll
-            for (int t = 0; t < 4; t++) { i32x2 v = rd((boff_base ^ (i << 4)) + STAGE_A + t * 8 * BN); bfrag[i][2 * t] = v[0]; bfrag[i][2 * t + 1] = v[1]; }
+        for (int i = 1; i < TN; i++) read_bfrag(i, 0);
+#pragma unroll
+        for (int d = 0; d < TN && d < NDMA; d++) issue_dma(d, 1, clamp_kb(kb_begin + 1));
+    }
+    for (int kb = kb_begin, it = 0; kb < kb_end; ++kb, ++it) {
+        const uint32_t cur = (it & 1) * STAGE, nxt = ((it + 1) & 1) * STAGE;
+        const int kn1 = clamp_kb(kb + 1), kn2 = clamp_kb(kb + 2);
+        const float s_last = s[TM - 1];                    // scale of the previous block's last m-tile (lagged folds)
+#pragma unroll
+        for (int j = 0; j < TM; j++) s[j] = sraw[j] * sb_cur;
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int t = 0; t < NMFMA + LAG; t++) {
-            if (t < NMFMA) {
-                const int j = t / TN, i = t % TN;
-                pring[t % PR] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                    bfrag[i], afrag[j & 1], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
-                asm volatile("" : "+v"(pring[t % PR]));      // anchor: the MFMA is issued here, not later
+        for (int t = 0; t < NMFMA; t++) {
+            const int j = t / TN, i = t % TN;
+            if (t == BAR_SLOT) {
+                // my DMA loads of the next stage have landed; after the barrier everyone's have, and everyone has
+                // finished reading the current stage (its last fragment was fetched one m-tile ago)
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                // b_scale of the next block was requested in slot 0. Touch it here, where the wait above has
+                // already covered it: the compiler then never waits for it later, behind the DMA loads it
+                // cannot see.
+                asm volatile("" : "+v"(sb_next));
+                __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
-                if (t < NDMA) issue_dma(t, nstage, kn);
-                if (j + 1 < TM && i == 0) {   // the next m-tile's fragment, a whole m-tile ahead of its use
-#pragma unroll
-                    for (int q = 0; q < 4; q++) {
-                        i32x2 v = rd((aoff_base ^ ((j + 1) << 4)) + q * 8 * BM);
-                        afrag[(j + 1) & 1][2 * q] = v[0];
-                        afrag[(j + 1) & 1][2 * q + 1] = v[1];
-                    }
+            }
+            if (t == 0) sb_next = SB[(size_t)kn1 * QN + nb + vzero];
+            pring[t % PR] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                bfrag[i], afrag[j & 1], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+            asm volatile("" : "+v"(pring[t % PR]));          // anchor: the MFMA is issued here, not later
+            __builtin_amdgcn_sched_barrier(0);
+            // LDS-DMA: the batch for block kb+1 (started in the previous iteration) continues in the first slots;
+            // the batch for block kb+2 starts right after the barrier
+            if (t + TN < NDMA) issue_dma(t + TN, (it + 1) & 1, kn1);
+            if (t >= BAR_SLOT && t - BAR_SLOT < NDMA) issue_dma(t - BAR_SLOT, it & 1, kn2);
+            // LDS -> registers
+            if (j + 1 < TM) {
+                if (i == 0) read_afrag((j + 1) & 1, j + 1, cur);      // a whole m-tile ahead of its use
+            } else {
+                read_bfrag(i, nxt);                                    // bfrag[i] is dead: refill for block kb+1
+                if (i == 0) {
+                    read_afrag(0, 0, nxt);
+                    read_scales(nxt);
                 }
             }
+            // lagged fold
             if (t >= LAG) {
-                const int u = t - LAG, j = u / TN, i = u % TN;
+                const int u = t - LAG, ju = u / TN, iu = u % TN;
 #pragma unroll
-                for (int e = 0; e < 4; e++) acc[j][i][e] = __builtin_fmaf(s[j], pring[u % PR][e], acc[j][i][e]);
-                asm volatile("" : "+v"(acc[j][i]));          // anchor: the fold happens in this slot
+                for (int e = 0; e < 4; e++) acc[ju][iu][e] = __builtin_fmaf(s[ju], pring[u % PR][e], acc[ju][iu][e]);
+                asm volatile("" : "+v"(acc[ju][iu]));        // anchor: the fold happens in this slot
+            } else {
+                const int u = NMFMA + t - LAG, ju = u / TN, iu = u % TN;   // tail of the previous K block
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[ju][iu][e] = __builtin_fmaf(s_last, pring[u % PR][e], acc[ju][iu][e]);
+                asm volatile("" : "+v"(acc[ju][iu]));
             }
             __builtin_amdgcn_sched_barrier(0);
         }
+        sb_cur = sb_next;
     }
-    // LDS-DMA writes of the last (redundant) prefetch must land before this workgroup's LDS can be handed on
+    // folds still owed by the last K block
+#pragma unroll
+    for (int t = 0; t < LAG; t++) {
+        const int u = NMFMA + t - LAG, ju = u / TN, iu = u % TN;
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc[ju][iu][e] = __builtin_fmaf(s[TM - 1], pring[u % PR][e], acc[ju][iu][e]);
+    }
+    // LDS-DMA writes of the last (redundant) prefetches must land before this workgroup's LDS can be handed on
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
     // ---- epilogue: lane holds C[m][n..n+3] per tile ----
