@@ -103,7 +103,18 @@ bool tiled_path_ok(const void *a, const void *b, const void *c, int m, int n) {
            ((uintptr_t)c % 8) == 0;
 }
 
-// Heuristic plan. Inputs: shape and CU count. The numbers come from sweeps on MI355X (256 CUs).
+// Plans measured on one MI355X by the tuner (python -m radeonflow_kernels_amd.tuner.gemm_tuner --all --emit).
+// The role of the reference's DISPATCH_GEMM table (src/gemm/gemm_launcher.cpp:229-259), except that a shape
+// outside the table is not an error: it gets the heuristic below.
+struct TunedPlan {
+    int m, n, k, variant, split_k, group_m;
+};
+const TunedPlan kTunedPlans[] = {
+    {0, 0, 0, 0, 1, 1},
+#include "tuned_plans.inc"
+};
+
+// Heuristic plan for shapes without a measured entry. Inputs: shape and CU count.
 void select_config(int m, int n, int k, int num_cu, bool tiled_ok, rf_gemm_config *out) {
     out->split_k = 1;
     out->group_m = 8;
@@ -111,6 +122,13 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, rf_gemm_confi
         out->variant = -1;
         return;
     }
+    for (const TunedPlan &p : kTunedPlans)
+        if (p.m == m && p.n == n && p.k == k && p.variant < kNumVariants && p.split_k <= k / rf::BK) {
+            out->variant = p.variant;
+            out->split_k = p.split_k;
+            out->group_m = p.group_m;
+            return;
+        }
     const int qk = k / rf::BK;
     int best = 1;
     long tiles_big = (long)ceil_div(m, 256) * ceil_div(n, 256);
