@@ -11,7 +11,6 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libgemm.so")
-CHECKER_PATH = os.path.join(LIB_DIR, "gemm_checker")
 
 # -packed-fp32-ops off: v_pk_{add,mul,fma}_f32 are kept out of the generated code on purpose.
 HIPCC_FLAGS = [
@@ -46,16 +45,22 @@ def build_lib(verbose=False):
 
 
 def build_checker(verbose=False):
-    src = os.path.join(CSRC, "gemm_checker.cpp")
-    if not os.path.exists(src):
-        return None
-    os.makedirs(LIB_DIR, exist_ok=True)
-    cmd = [hipcc(), "-O2", "-std=c++17", "-fopenmp", "-o", CHECKER_PATH, src, "-ldl",
-           "-Wl,-rpath,$ORIGIN"]
-    out = _run(cmd)
-    if verbose and out:
-        print(out)
-    return CHECKER_PATH
+    """tests/checker/gemm_checker: native harness (test infrastructure; links the C oracle, dlopens libgemm.so)."""
+    root = os.path.dirname(HERE)
+    src = os.path.join(root, "tests", "checker", "gemm_checker.cpp")
+    oracle = os.path.join(root, "oracle", "fp8_blockscale_oracle.c")
+    out = os.path.join(root, "tests", "checker", "gemm_checker")
+    obj = os.path.join(root, "tests", "checker", "oracle.o")
+    _run(["gcc", "-O2", "-fopenmp", "-std=c11", "-ffp-contract=off", "-c", oracle, "-o", obj])
+    rocm = os.path.dirname(os.path.dirname(os.path.realpath(hipcc())))
+    # host-only program: plain g++ against the HIP runtime library
+    cmd = ["g++", "-O2", "-std=c++17", "-fopenmp", "-D__HIP_PLATFORM_AMD__", "-I" + os.path.join(rocm, "include"),
+           "-o", out, src, obj, "-L" + os.path.join(rocm, "lib"), "-lamdhip64", "-ldl", "-lm",
+           "-Wl,-rpath," + os.path.join(rocm, "lib"), "-Wl,-rpath,$ORIGIN/../../radeonflow_kernels_amd/lib"]
+    res = _run(cmd)
+    if verbose and res:
+        print(res)
+    return out
 
 
 def build_all(verbose=False):

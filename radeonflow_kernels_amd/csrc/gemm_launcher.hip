@@ -330,6 +330,7 @@ void run(void *a, void *b, void *as, void *bs, void *c, int m, int n, int k, Per
     if (rc != RF_OK) {
         if (rc == RF_ERR_BAD_SHAPE) printf("Error: Unsupported shape M=%d, K=%d, N=%d\n", m, k, n);
         fprintf(stderr, "Kernel execution failed.\n%s\n", g_last_error.c_str());
+        fflush(stdout);
         abort();
     }
     if (job) {

@@ -1,0 +1,68 @@
+"""CPU-only checks of the C ABI: libgemm.so loads, exports what include/rf_gemm.h declares, and rejects bad
+arguments before touching a device."""
+import ctypes
+import os
+import re
+import subprocess
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "rf_gemm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(run|rf_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from radeonflow_kernels_amd import gemm
+    lib = ctypes.CDLL(gemm.LIB_PATH)
+    names = _declared_functions()
+    assert "run" in names and "rf_fp8_gemm" in names and len(names) >= 10
+    for n in names:
+        assert hasattr(lib, n), "libgemm.so does not export %s" % n
+    assert sorted(gemm.EXPORTS) == names
+
+
+def test_perf_metrics_layout_matches_the_reference_struct():
+    from radeonflow_kernels_amd.gemm import PerfMetrics, PerfMetricEntry, GemmConfig
+    assert ctypes.sizeof(PerfMetricEntry) == 28
+    assert ctypes.sizeof(PerfMetrics) == 4 + 20 * 28 == 564
+    assert PerfMetrics.entries.offset == 4
+    assert PerfMetricEntry.time.offset == 20 and PerfMetricEntry.gflops.offset == 24
+    assert ctypes.sizeof(GemmConfig) == 12
+
+
+def test_status_codes_without_a_device():
+    from radeonflow_kernels_amd import gemm
+    L = gemm.lib()
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.addressof(buf)
+    assert L.rf_fp8_gemm(p, p, p, p, p, 16, 16, 100, None) == 1          # K not a multiple of 128
+    assert b"K=100" in L.rf_gemm_last_error()
+    assert L.rf_fp8_gemm(p, p, p, p, p, 16, 16, 0, None) == 1
+    assert L.rf_fp8_gemm(p, p, p, p, p, -1, 16, 128, None) == 1
+    assert L.rf_fp8_gemm(None, p, p, p, p, 16, 16, 128, None) == 2        # null pointer
+    assert L.rf_gemm_num_variants() >= 1
+    info = [ctypes.c_int() for _ in range(5)]
+    assert L.rf_gemm_variant_info(0, *[ctypes.byref(x) for x in info]) == 0
+    assert info[0].value % 16 == 0 and info[4].value <= 160 * 1024        # fits the 160 KiB LDS of a gfx950 CU
+    assert L.rf_gemm_variant_info(999, *[ctypes.byref(x) for x in info]) == 4
+
+
+def test_run_aborts_on_an_unsupported_shape_like_the_reference_launcher():
+    code = ("import ctypes,sys; sys.path.insert(0,%r); from radeonflow_kernels_amd import gemm; L=gemm.lib(); "
+            "b=ctypes.create_string_buffer(64); p=ctypes.addressof(b); L.run(p,p,p,p,p,64,64,100,None,None)" % ROOT)
+    r = subprocess.run([sys.executable, "-c", code], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
+    assert r.returncode == -6                                              # SIGABRT
+    assert "Unsupported shape M=64, K=100, N=64" in r.stdout
+
+
+def test_python_mirror_rejects_cpu_tensors_and_wrong_layouts():
+    import pytest
+    import torch
+    import radeonflow_kernels_amd as rfk
+    a = torch.zeros((16, 128), dtype=torch.uint8).view(torch.float8_e4m3fn)
+    with pytest.raises(ValueError):
+        rfk.fp8_mm(a, a, torch.zeros(16, 1), torch.zeros(1, 1), torch.zeros((16, 16), dtype=torch.bfloat16))
