@@ -44,6 +44,8 @@ typedef struct rf_gemm_config {
     int variant;      /* index into the variant table, see rf_gemm_variant_info(); -1 = bounds-checked kernel */
     int split_k;      /* >= 1; K blocks are divided over this many partial sums */
     int group_m;      /* tile-order grouping along M for L2 reuse (>=1) */
+    int stream_k;     /* 1: persistent grid, one workgroup per CU, equal shares of the tile x K-block work line;
+                         needs split_k == 1 and at least as many tiles as CUs. 0: one workgroup per tile */
 } rf_gemm_config;
 
 /* Drop-in for the reference's launcher entry (src/gemm/gemm_launcher.cpp:182-184):

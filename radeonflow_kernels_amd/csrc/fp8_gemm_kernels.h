@@ -62,10 +62,13 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 // logical ids in groups of `group_m` tile rows so that the tiles resident on one XCD at a time
 // form a compact patch that re-uses A rows and B columns from that XCD's L2.
 __device__ __forceinline__ void tile_of_block(int bid, int nblocks, int tiles_m, int tiles_n, int group_m,
-                                              int &tile_m, int &tile_n) {
-    int xcd = bid % NUM_XCD, idx = bid / NUM_XCD;
-    int per = nblocks / NUM_XCD, rem = nblocks % NUM_XCD;
-    int id = xcd * per + (xcd < rem ? xcd : rem) + idx;
+                                              bool xcd_remap, int &tile_m, int &tile_n) {
+    int id = bid;
+    if (xcd_remap) {
+        int xcd = bid % NUM_XCD, idx = bid / NUM_XCD;
+        int per = nblocks / NUM_XCD, rem = nblocks % NUM_XCD;
+        id = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    }
     int group_sz = group_m * tiles_n;
     int grp = id / group_sz;
     int first_m = grp * group_m;
@@ -75,17 +78,24 @@ __device__ __forceinline__ void tile_of_block(int bid, int nblocks, int tiles_m,
     tile_n = in_grp / rows;
 }
 
-// ---------------------------------------------------------------------------------------------
-// Tiled MFMA kernel. PARTIAL=false: writes bf16 C. PARTIAL=true: writes fp32 partial sums of the
-// K range of split blockIdx.y to ws[split][M][N].
-// Requirements checked by the host: M%16==0, N%16==0, M>=16, N>=16, a/b 16-byte aligned,
-// c 8-byte aligned, K%128==0.
-// ---------------------------------------------------------------------------------------------
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool PARTIAL>
-__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_tile(
+// Geometry of one kernel variant.
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_>
+struct TileGeom {
+    static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+    static constexpr int NW = WAVES_M * WAVES_N, NT = NW * 64;
+    static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 16, TN = WN / 16;
+    static constexpr int STAGE = BK * BM + BK * BN + BM * 4;      // A rows, B rows, a_scale
+    static constexpr int LDS_BYTES = 2 * STAGE + 16;              // two stages + a 16-byte mailbox
+};
+
+// Accumulates into acc the contribution of K blocks [kb_begin, kb_end) to the BM x BN tile at (m0, n0).
+// All waves of the workgroup call it together. On return every LDS-DMA load has landed, but other waves may still
+// be reading LDS: a barrier is needed before LDS is written again.
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+__device__ __forceinline__ void tile_mainloop(
     const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
-    const float *__restrict__ SB, void *__restrict__ Cout, int M, int N, int K, int kb_per_split,
-    int tiles_m, int tiles_n, int group_m) {
+    const float *__restrict__ SB, int M, int N, int m0, int n0, int kb_begin, int kb_end, uint8_t *lds,
+    f32x4 (&acc)[BM / WAVES_M / 16][BN / WAVES_N / 16]) {
     constexpr int NW = WAVES_M * WAVES_N;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     constexpr int TM = WM / 16, TN = WN / 16;
@@ -100,20 +110,13 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
     constexpr int CPR_A = BM / 16, CPR_B = BN / 16;          // 16-byte chunks per LDS row
     constexpr int RPI_A = 1024 / BM, RPI_B = 1024 / BN;      // rows per load instruction
 
-    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
-
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int L = lane & 15, g = lane >> 4;
     const int wm = wave % WAVES_M, wn = wave / WAVES_M;
 
-    int tile_m, tile_n;
-    tile_of_block(blockIdx.x, tiles_m * tiles_n, tiles_m, tiles_n, group_m, tile_m, tile_n);
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int QK = K / BK, QN = (N + 127) / 128;
-    const int kb_begin = blockIdx.y * kb_per_split;
-    const int kb_end = kb_begin + kb_per_split < QK ? kb_begin + kb_per_split : QK;
+    const int QN = (N + 127) / 128;
 
     // ---- global -> LDS: per-lane source offsets inside one K block (rows k_local, swizzled chunk) ----
     // Load instruction i of this wave covers rows (wave*INST + i)*RPI .. +RPI-1. Its per-lane offset differs from
@@ -164,24 +167,32 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
     // the LDS destination of the instruction (lane l lands at M0 + 16*l, or M0 + 4*l for the dword form).
     const uint32_t lds_base = (uint32_t)(uintptr_t)(RF_LDS uint8_t *)lds;
     constexpr int NDMA = INST_A + INST_B + 1;
-    // DMA instruction `d` of this wave for K block kb into `stage`: A rows, then B rows, then the scales
-    auto issue_dma = [&](int d, int stage, int kb) {
+    // DMA instruction d of this wave: A rows (d < INST_A), then B rows, then the scales. Its global source for K
+    // block kb is dma_src(d, kb); its LDS destination inside a stage is fixed. In the loop each instruction keeps a
+    // running source pointer (one 64-bit scalar add per K block) instead of recomputing products.
+    const uint32_t lds_dst_a = lds_base + wave * (INST_A * 1024), lds_dst_b = lds_base + STAGE_A + wave * (INST_B * 1024),
+                   lds_dst_s = lds_base + STAGE_A + STAGE_B + wave * 256;
+    auto dma_src = [&](int d, int kb) -> const uint8_t * {
+        if (d < INST_A) return A + ((size_t)kb * BK + (size_t)(wave * INST_A + d) * RPI_A) * M;
+        if (d < INST_A + INST_B) return B + ((size_t)kb * BK + (size_t)(wave * INST_B + (d - INST_A)) * RPI_B) * N;
+        return (const uint8_t *)(SA + (size_t)kb * M);
+    };
+    auto dma_step = [&](int d) -> size_t {       // bytes from one K block to the next
+        return d < INST_A ? (size_t)BK * M : d < INST_A + INST_B ? (size_t)BK * N : (size_t)M * 4;
+    };
+    auto issue_dma = [&](int d, uint32_t stage_off, const uint8_t *src) {
         if (d < INST_A) {
-            const uint8_t *ak = A + ((size_t)kb * BK + (size_t)(wave * INST_A + d) * RPI_A) * M;
-            const uint32_t dst = lds_base + stage * STAGE + (wave * INST_A + d) * 1024;
-            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                         :: "v"(goff_a[cls_a(d < INST_A ? d : 0)]), "s"(ak), "s"(dst) : "memory");
+            asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                         :: "v"(goff_a[cls_a(d < INST_A ? d : 0)]), "s"(src), "s"(stage_off + lds_dst_a), "n"(d * 1024)
+                         : "memory", "scc");
         } else if (d < INST_A + INST_B) {
             const int e = d - INST_A < INST_B ? d - INST_A : 0;
-            const uint8_t *bk = B + ((size_t)kb * BK + (size_t)(wave * INST_B + e) * RPI_B) * N;
-            const uint32_t dst = lds_base + stage * STAGE + STAGE_A + (wave * INST_B + e) * 1024;
-            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                         :: "v"(goff_b[cls_b(e >= 0 ? e : 0)]), "s"(bk), "s"(dst) : "memory");
+            asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                         :: "v"(goff_b[cls_b(e >= 0 ? e : 0)]), "s"(src), "s"(stage_off + lds_dst_b), "n"(e * 1024)
+                         : "memory", "scc");
         } else if (wave < NSC) {
-            const float *sk = SA + (size_t)kb * M;
-            const uint32_t dst = lds_base + stage * STAGE + STAGE_A + STAGE_B + wave * 256;
             asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
-                         :: "v"(goff_s), "s"(sk), "s"(dst) : "memory");
+                         :: "v"(goff_s), "s"(src), "s"(stage_off + lds_dst_s) : "memory");
         }
     };
 
@@ -198,7 +209,6 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
     int nb = (n0 + wn * WN) >> 7;
     if (nb > QN - 1) nb = QN - 1;
 
-    f32x4 acc[TM][TN];
 #pragma unroll
     for (int j = 0; j < TM; j++)
 #pragma unroll
@@ -267,7 +277,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
     if (kb_begin < kb_end) {
         // prologue: stage 0 <- first K block, then its first operands; stage 1 <- second K block
 #pragma unroll
-        for (int d = 0; d < NDMA; d++) issue_dma(d, 0, kb_begin);
+        for (int d = 0; d < NDMA; d++) issue_dma(d, 0, dma_src(d, kb_begin));
         sb_cur = SB[(size_t)kb_begin * QN + nb + vzero];
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         asm volatile("" : "+v"(sb_cur));
@@ -278,11 +288,17 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
 #pragma unroll
         for (int i = 1; i < TN; i++) read_bfrag(i, 0);
 #pragma unroll
-        for (int d = 0; d < TN && d < NDMA; d++) issue_dma(d, 1, clamp_kb(kb_begin + 1));
+        for (int d = 0; d < TN && d < NDMA; d++) issue_dma(d, STAGE, dma_src(d, clamp_kb(kb_begin + 1)));
     }
+    // running DMA sources: instructions d >= TN are issued for block kb+1 in the first slots of iteration kb,
+    // instructions d < TN for block kb+2 in its last slots (blocks past the end are clamped to the last one)
+    const uint8_t *dsrc[NDMA];
+#pragma unroll
+    for (int d = 0; d < NDMA; d++) dsrc[d] = dma_src(d, clamp_kb(kb_begin + (d < TN ? 2 : 1)));
     for (int kb = kb_begin, it = 0; kb < kb_end; ++kb, ++it) {
         const uint32_t cur = (it & 1) * STAGE, nxt = ((it + 1) & 1) * STAGE;
-        const int kn1 = clamp_kb(kb + 1), kn2 = clamp_kb(kb + 2);
+        const int kn1 = clamp_kb(kb + 1);
+        const bool adv1 = kb + 2 <= kb_last, adv2 = kb + 3 <= kb_last;   // does the next iteration move on a block?
         const float s_last = s[TM - 1];                    // scale of the previous block's last m-tile (lagged folds)
 #pragma unroll
         for (int j = 0; j < TM; j++) s[j] = sraw[j] * sb_cur;
@@ -308,8 +324,14 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
             __builtin_amdgcn_sched_barrier(0);
             // LDS-DMA: the batch for block kb+1 (started in the previous iteration) continues in the first slots;
             // the batch for block kb+2 starts right after the barrier
-            if (t + TN < NDMA) issue_dma(t + TN, (it + 1) & 1, kn1);
-            if (t >= BAR_SLOT && t - BAR_SLOT < NDMA) issue_dma(t - BAR_SLOT, it & 1, kn2);
+            if (t + TN < NDMA) {
+                issue_dma(t + TN, nxt, dsrc[t + TN]);
+                dsrc[t + TN] += adv1 ? dma_step(t + TN) : 0;
+            }
+            if (t >= BAR_SLOT && t - BAR_SLOT < NDMA && t - BAR_SLOT < TN) {
+                issue_dma(t - BAR_SLOT, cur, dsrc[t - BAR_SLOT]);
+                dsrc[t - BAR_SLOT] += adv2 ? dma_step(t - BAR_SLOT) : 0;
+            }
             // LDS -> registers
             if (j + 1 < TM) {
                 if (i == 0) read_afrag((j + 1) & 1, j + 1, cur);      // a whole m-tile ahead of its use
@@ -346,26 +368,176 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
     // LDS-DMA writes of the last (redundant) prefetches must land before this workgroup's LDS can be handed on
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-    // ---- epilogue: lane holds C[m][n..n+3] per tile ----
+}
+
+// Stores a wave's accumulators: bf16 into C (masked at the M and N edges), or fp32 into a BM x BN workspace tile.
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+__device__ __forceinline__ void store_tile_bf16(const f32x4 (&acc)[BM / WAVES_M / 16][BN / WAVES_N / 16],
+                                                uint16_t *__restrict__ C, int M, int N, int m0, int n0) {
+    using G = TileGeom<BM, BN, WAVES_M, WAVES_N>;
+    // the opaque zero keeps this address arithmetic below the main loop: hoisted above it, it would cost the
+    // loop dozens of registers
+    int vz;
+    asm volatile("v_mov_b32 %0, 0" : "=v"(vz));
+    const int lane = (threadIdx.x & 63) + vz, wave = threadIdx.x >> 6, L = lane & 15, g = lane >> 4;
+    const int wm = wave % WAVES_M, wn = wave / WAVES_M;
 #pragma unroll
-    for (int j = 0; j < TM; j++) {
-        const int m = m0 + wm * WM + 16 * j + L;
+    for (int j = 0; j < G::TM; j++) {
+        const int m = m0 + wm * G::WM + 16 * j + L;
 #pragma unroll
-        for (int i = 0; i < TN; i++) {
-            const int n = n0 + wn * WN + 16 * i + 4 * g;
+        for (int i = 0; i < G::TN; i++) {
+            const int n = n0 + wn * G::WN + 16 * i + 4 * g;      // lane holds C[m][n..n+3]
             if (m < M && n < N) {
-                if constexpr (PARTIAL) {
-                    float *ws = (float *)Cout + ((size_t)blockIdx.y * M + m) * N + n;
-                    *(f32x4 *)ws = acc[j][i];
-                } else {
-                    uint16_t *c = (uint16_t *)Cout + (size_t)m * N + n;
-                    uint2 v;
-                    v.x = pack_bf16x2(acc[j][i][0], acc[j][i][1]);
-                    v.y = pack_bf16x2(acc[j][i][2], acc[j][i][3]);
-                    *(uint2 *)c = v;
-                }
+                uint2 v;
+                v.x = pack_bf16x2(acc[j][i][0], acc[j][i][1]);
+                v.y = pack_bf16x2(acc[j][i][2], acc[j][i][3]);
+                *(uint2 *)(C + (size_t)m * N + n) = v;
             }
         }
+    }
+}
+
+// fp32 tile with leading dimension ld; rows < m_lim and cols < n_lim are written (limits relative to the tile).
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+__device__ __forceinline__ void store_tile_f32(const f32x4 (&acc)[BM / WAVES_M / 16][BN / WAVES_N / 16],
+                                               float *__restrict__ t, size_t ld, int m_lim, int n_lim) {
+    using G = TileGeom<BM, BN, WAVES_M, WAVES_N>;
+    int vz;                                  // see store_tile_bf16
+    asm volatile("v_mov_b32 %0, 0" : "=v"(vz));
+    const int lane = (threadIdx.x & 63) + vz, wave = threadIdx.x >> 6, L = lane & 15, g = lane >> 4;
+    const int wm = wave % WAVES_M, wn = wave / WAVES_M;
+#pragma unroll
+    for (int j = 0; j < G::TM; j++) {
+        const int m = wm * G::WM + 16 * j + L;
+#pragma unroll
+        for (int i = 0; i < G::TN; i++) {
+            const int n = wn * G::WN + 16 * i + 4 * g;
+            if (m < m_lim && n < n_lim) *(f32x4 *)(t + (size_t)m * ld + n) = acc[j][i];
+        }
+    }
+}
+
+// Partial tiles exchanged between workgroups of the stream-K grid. The two workgroups may sit on different XCDs,
+// whose L2 caches are not coherent with each other. Instead of device-wide fences (which write back and invalidate
+// a whole L2, throwing away the A/B tiles every other workgroup on the XCD is re-using), each access carries system
+// scope itself: relaxed 64-bit atomic stores write through to memory, relaxed atomic loads bypass the caches.
+// Layout is register order (tile (j,i) of wave w at ((w*TM + j)*TN + i)*256 floats, lane l at +4l): every store
+// instruction covers 1 KiB of contiguous memory; the only reader is a workgroup with the same thread mapping.
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool ACCUMULATE_FROM>
+__device__ __forceinline__ void exchange_tile_f32(f32x4 (&acc)[BM / WAVES_M / 16][BN / WAVES_N / 16], float *t) {
+    using G = TileGeom<BM, BN, WAVES_M, WAVES_N>;
+    int vz;                                  // see store_tile_bf16
+    asm volatile("v_mov_b32 %0, 0" : "=v"(vz));
+    uint64_t *q = (uint64_t *)(t + ((size_t)(threadIdx.x >> 6) * (G::TM * G::TN) * 64 + (threadIdx.x & 63) + vz) * 4);
+#pragma unroll
+    for (int j = 0; j < G::TM; j++) {
+#pragma unroll
+        for (int i = 0; i < G::TN; i++) {
+            if constexpr (ACCUMULATE_FROM) {
+                f32x2 lo = __builtin_bit_cast(f32x2, __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM));
+                f32x2 hi = __builtin_bit_cast(f32x2, __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM));
+                acc[j][i][0] += lo[0]; acc[j][i][1] += lo[1]; acc[j][i][2] += hi[0]; acc[j][i][3] += hi[1];
+            } else {
+                f32x2 lo = {acc[j][i][0], acc[j][i][1]}, hi = {acc[j][i][2], acc[j][i][3]};
+                __hip_atomic_store(q, __builtin_bit_cast(uint64_t, lo), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                __hip_atomic_store(q + 1, __builtin_bit_cast(uint64_t, hi), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
+            q += 128;                        // next tile: 64 lanes x 16 bytes further
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// One workgroup per (tile, K split). PARTIAL=false: writes bf16 C. PARTIAL=true: writes the fp32 partial sums of
+// the K range of split blockIdx.y to ws[split][M][N] (summed by reduce_splitk_bf16).
+// Requirements checked by the host: M%16==0, N%16==0, M>=16, N>=16, a/b 16-byte aligned,
+// c 8-byte aligned, K%128==0.
+// ---------------------------------------------------------------------------------------------
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool PARTIAL>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_tile(
+    const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
+    const float *__restrict__ SB, void *__restrict__ Cout, int M, int N, int K, int kb_per_split,
+    int tiles_m, int tiles_n, int group_m) {
+    using G = TileGeom<BM, BN, WAVES_M, WAVES_N>;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    int tile_m, tile_n;
+    tile_of_block(blockIdx.x, tiles_m * tiles_n, tiles_m, tiles_n, group_m, true, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int QK = K / BK;
+    const int kb_begin = blockIdx.y * kb_per_split;
+    const int kb_end = kb_begin + kb_per_split < QK ? kb_begin + kb_per_split : QK;
+    f32x4 acc[G::TM][G::TN];
+    tile_mainloop<BM, BN, WAVES_M, WAVES_N>(A, B, SA, SB, M, N, m0, n0, kb_begin, kb_end, lds, acc);
+    if constexpr (PARTIAL)
+        store_tile_f32<BM, BN, WAVES_M, WAVES_N>(acc, (float *)Cout + ((size_t)blockIdx.y * M + m0) * N + n0, N, M - m0,
+                                                 N - n0);
+    else
+        store_tile_bf16<BM, BN, WAVES_M, WAVES_N>(acc, (uint16_t *)Cout, M, N, m0, n0);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Stream-K: a persistent grid of P workgroups (one per CU). The T tiles x QK K-blocks are laid out as one line of
+// work units and cut into P equal contiguous ranges, so every CU gets the same number of MFMAs whatever T is
+// (432 tiles on 256 CUs is 1.69 tiles each, not 2). A workgroup walks its range tile by tile. A tile whose K
+// range is shared by several workgroups is finished by whichever of them arrives last: each one stores its fp32
+// partial tile to its workspace slot with write-through stores and bumps the tile's counter; the one that
+// reads count == parts-1 adds the other partials and writes bf16. Nobody waits for anybody, so there is nothing to
+// deadlock, and the last arriver resets the counter: the counters are zero again when the kernel ends.
+// Used only when every range is at least QK units long (T >= P), so a split tile has exactly 2 contributors.
+// ws: tile_count[T] (unsigned, zero on entry), then at byte offset ws_slots_off 2*P slots of BM*BN floats.
+// ---------------------------------------------------------------------------------------------
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_streamk(
+    const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
+    const float *__restrict__ SB, uint16_t *__restrict__ C, int M, int N, int K, int tiles_m, int tiles_n, int group_m,
+    unsigned *__restrict__ tile_count, float *__restrict__ slots) {
+    using G = TileGeom<BM, BN, WAVES_M, WAVES_N>;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    volatile unsigned *mailbox = (volatile unsigned *)(lds + 2 * G::STAGE);
+    const int P = gridDim.x, QK = K / BK;
+    const long long U = (long long)tiles_m * tiles_n * QK;
+    // workgroups are dealt round-robin to the XCDs: give each XCD a contiguous band of the unit line
+    const int xcd = blockIdx.x % NUM_XCD, idx = blockIdx.x / NUM_XCD, per = P / NUM_XCD, rem = P % NUM_XCD;
+    const int slot = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    auto lo_of = [&](int s) { return (long long)s * U / P; };
+    auto slot_of = [&](long long u) { return (int)((((u + 1) * P) - 1) / U); };   // largest s with lo_of(s) <= u
+    const long long lo = lo_of(slot), hi = lo_of(slot + 1);
+    for (long long u = lo; u < hi;) {
+        const int tile = (int)(u / QK);
+        const long long tq = (long long)tile * QK;
+        const int kb0 = (int)(u - tq);
+        const int kb1 = hi - tq < QK ? (int)(hi - tq) : QK;
+        int tile_m, tile_n;
+        tile_of_block(tile, tiles_m * tiles_n, tiles_m, tiles_n, group_m, false, tile_m, tile_n);
+        const int m0 = tile_m * BM, n0 = tile_n * BN;
+        f32x4 acc[G::TM][G::TN];
+        __syncthreads();                     // every wave is done with LDS (previous segment, or the mailbox)
+        tile_mainloop<BM, BN, WAVES_M, WAVES_N>(A, B, SA, SB, M, N, m0, n0, kb0, kb1, lds, acc);
+        bool write_c = (kb0 == 0 && kb1 == QK);
+        if (!write_c) {
+            // the host only launches this kernel with T >= P, so a tile has exactly two contributors: the workgroup
+            // whose range ends inside it and the next one
+            const int s_first = slot_of(tq);
+            const int other = slot == s_first ? slot + 1 : slot - 1;
+            // a contributor's slot: 2*s for the first segment of its range, 2*s+1 when the tile starts before its range
+            auto slot_ptr = [&](int s) { return slots + (size_t)(2 * s + (lo_of(s) < tq ? 1 : 0)) * (BM * BN); };
+            exchange_tile_f32<BM, BN, WAVES_M, WAVES_N, false>(acc, slot_ptr(slot));
+            // the write-through stores are acknowledged (vmcnt) once they are at the coherence point; only then may
+            // the counter move
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (threadIdx.x == 0)
+                *mailbox = __hip_atomic_fetch_add(tile_count + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+            if (*mailbox == 1u) {            // the other contributor arrived first: I finish the tile
+                exchange_tile_f32<BM, BN, WAVES_M, WAVES_N, true>(acc, slot_ptr(other));
+                if (threadIdx.x == 0)        // ready for the next launch
+                    __hip_atomic_store(tile_count + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                write_c = true;
+            }
+        }
+        if (write_c) store_tile_bf16<BM, BN, WAVES_M, WAVES_N>(acc, C, M, N, m0, n0);
+        u = tq + kb1;
     }
 }
 

@@ -34,15 +34,19 @@ int fail(int code, const std::string &msg) {
 // ---- variant table -------------------------------------------------------------------------
 typedef void (*tile_kernel_t)(const uint8_t *, const uint8_t *, const float *, const float *, void *, int, int, int,
                               int, int, int, int);
+typedef void (*streamk_kernel_t)(const uint8_t *, const uint8_t *, const float *, const float *, uint16_t *, int, int,
+                                 int, int, int, int, unsigned *, float *);
 struct Variant {
     int bm, bn, waves_m, waves_n;
     tile_kernel_t direct, partial;
-    int lds_bytes() const { return 2 * (rf::BK * (bm + bn) + 4 * bm); }
+    streamk_kernel_t streamk;
+    int lds_bytes() const { return 2 * (rf::BK * (bm + bn) + 4 * bm) + 16; }
     int threads() const { return waves_m * waves_n * 64; }
 };
 #define RF_VARIANT(BM, BN, WM, WN)                                                         \
     Variant { BM, BN, WM, WN, rf::gemm_fp8_blockscale_tile<BM, BN, WM, WN, false>,         \
-              rf::gemm_fp8_blockscale_tile<BM, BN, WM, WN, true> }
+              rf::gemm_fp8_blockscale_tile<BM, BN, WM, WN, true>,                          \
+              rf::gemm_fp8_blockscale_streamk<BM, BN, WM, WN> }
 const Variant kVariants[] = {
     RF_VARIANT(256, 256, 2, 4),   // 0: 8 waves, wave tile 128(m) x 64(n), 128 KiB LDS
     RF_VARIANT(128, 128, 2, 2),   // 1: 4 waves, wave tile 64 x 64, 64 KiB LDS (2 workgroups per CU)
@@ -57,6 +61,7 @@ struct State {
     std::mutex mu;
     float *ws = nullptr;
     size_t ws_bytes = 0;
+    unsigned *tile_count = nullptr;      // stream-K arrival counters, zero between launches
     bool attrs_set = false;
     int num_cu = 0;
     std::vector<std::pair<hipEvent_t, hipEvent_t>> free_events;
@@ -78,6 +83,7 @@ int ensure_device_info(State &s) {
     for (const Variant &v : kVariants) {
         RF_HIP(hipFuncSetAttribute((const void *)v.direct, hipFuncAttributeMaxDynamicSharedMemorySize, v.lds_bytes()));
         RF_HIP(hipFuncSetAttribute((const void *)v.partial, hipFuncAttributeMaxDynamicSharedMemorySize, v.lds_bytes()));
+        RF_HIP(hipFuncSetAttribute((const void *)v.streamk, hipFuncAttributeMaxDynamicSharedMemorySize, v.lds_bytes()));
     }
     s.attrs_set = true;
     return RF_OK;
@@ -96,6 +102,15 @@ int ensure_workspace(State &s, size_t bytes) {
     return RF_OK;
 }
 
+constexpr int kMaxStreamKTiles = 16384;
+
+int ensure_tile_counters(State &s) {
+    if (s.tile_count) return RF_OK;
+    RF_HIP(hipMalloc((void **)&s.tile_count, kMaxStreamKTiles * sizeof(unsigned)));
+    RF_HIP(hipMemset(s.tile_count, 0, kMaxStreamKTiles * sizeof(unsigned)));
+    return RF_OK;
+}
+
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 bool tiled_path_ok(const void *a, const void *b, const void *c, int m, int n) {
@@ -107,10 +122,10 @@ bool tiled_path_ok(const void *a, const void *b, const void *c, int m, int n) {
 // The role of the reference's DISPATCH_GEMM table (src/gemm/gemm_launcher.cpp:229-259), except that a shape
 // outside the table is not an error: it gets the heuristic below.
 struct TunedPlan {
-    int m, n, k, variant, split_k, group_m;
+    int m, n, k, variant, split_k, group_m, stream_k;
 };
 const TunedPlan kTunedPlans[] = {
-    {0, 0, 0, 0, 1, 1},
+    {0, 0, 0, 0, 1, 1, 0},
 #include "tuned_plans.inc"
 };
 
@@ -118,6 +133,7 @@ const TunedPlan kTunedPlans[] = {
 void select_config(int m, int n, int k, int num_cu, bool tiled_ok, rf_gemm_config *out) {
     out->split_k = 1;
     out->group_m = 8;
+    out->stream_k = 0;
     if (!tiled_ok) {
         out->variant = -1;
         return;
@@ -127,12 +143,17 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, rf_gemm_confi
             out->variant = p.variant;
             out->split_k = p.split_k;
             out->group_m = p.group_m;
+            out->stream_k = p.stream_k;
             return;
         }
     const int qk = k / rf::BK;
     int best = 1;
     long tiles_big = (long)ceil_div(m, 256) * ceil_div(n, 256);
-    if (tiles_big >= num_cu) best = 0;
+    if (tiles_big >= num_cu) {
+        // stream_k stays off here: cutting tiles at arbitrary K blocks puts the workgroups of an XCD at different K
+        // positions, they stop sharing A/B lines in L2, and that costs more than the uneven last round (measured)
+        best = 0;
+    }
     out->variant = best;
     const Variant &v = kVariants[best];
     long tiles = (long)ceil_div(m, v.bm) * ceil_div(n, v.bn);
@@ -162,8 +183,15 @@ int launch(const void *a, const void *b, const float *as, const float *bs, void 
     if (user_cfg) {
         cfg = *user_cfg;
         if (cfg.variant >= kNumVariants || cfg.variant < -1 || cfg.split_k < 1 || cfg.group_m < 1 ||
-            cfg.split_k > k / rf::BK || (cfg.variant >= 0 && !tiled_ok) || (cfg.variant < 0 && cfg.split_k != 1))
+            cfg.split_k > k / rf::BK || (cfg.variant >= 0 && !tiled_ok) || (cfg.variant < 0 && cfg.split_k != 1) ||
+            (cfg.stream_k != 0 && (cfg.variant < 0 || cfg.split_k != 1)))
             return fail(RF_ERR_BAD_CONFIG, "configuration not usable for this shape");
+        if (cfg.stream_k != 0) {
+            const Variant &sv = kVariants[cfg.variant];
+            const long t = (long)ceil_div(m, sv.bm) * ceil_div(n, sv.bn);
+            if (t < s.num_cu || t > kMaxStreamKTiles)
+                return fail(RF_ERR_BAD_CONFIG, "stream_k needs at least as many tiles as compute units");
+        }
     } else {
         select_config(m, n, k, s.num_cu, tiled_ok, &cfg);
     }
@@ -183,6 +211,17 @@ int launch(const void *a, const void *b, const float *as, const float *bs, void 
     const int splits = ceil_div(qk, kb_per_split);          // every split owns at least one K block
     dim3 grid(tiles_m * tiles_n, splits);
     dim3 block(v.threads());
+    if (cfg.stream_k != 0) {
+        const int P = s.num_cu;
+        rc = ensure_tile_counters(s);
+        if (rc != RF_OK) return rc;
+        rc = ensure_workspace(s, (size_t)2 * P * v.bm * v.bn * sizeof(float));
+        if (rc != RF_OK) return rc;
+        hipLaunchKernelGGL(v.streamk, dim3(P), block, v.lds_bytes(), stream, (const uint8_t *)a, (const uint8_t *)b, as,
+                           bs, (uint16_t *)c, m, n, k, tiles_m, tiles_n, cfg.group_m, s.tile_count, s.ws);
+        RF_HIP(hipGetLastError());
+        return RF_OK;
+    }
     if (splits == 1) {
         hipLaunchKernelGGL(v.direct, grid, block, v.lds_bytes(), stream, (const uint8_t *)a, (const uint8_t *)b, as, bs,
                            c, m, n, k, kb_per_split, tiles_m, tiles_n, cfg.group_m);
@@ -265,7 +304,12 @@ int rf_gemm_variant_info(int variant, int *block_m, int *block_n, int *waves_m, 
 
 size_t rf_gemm_workspace_bytes(int m, int n, int k) {
     rf_gemm_config cfg;
-    if (rf_gemm_select_config(m, n, k, &cfg) != RF_OK || cfg.variant < 0 || cfg.split_k <= 1) return 0;
+    if (rf_gemm_select_config(m, n, k, &cfg) != RF_OK || cfg.variant < 0) return 0;
+    if (cfg.stream_k != 0) {
+        State &s = state();
+        return (size_t)2 * s.num_cu * kVariants[cfg.variant].bm * kVariants[cfg.variant].bn * sizeof(float);
+    }
+    if (cfg.split_k <= 1) return 0;
     const int qk = k / rf::BK;
     const int kb_per_split = ceil_div(qk, cfg.split_k);
     return (size_t)m * n * sizeof(float) * ceil_div(qk, kb_per_split);
@@ -289,6 +333,8 @@ void rf_gemm_destroy(void) {
     }
     s.ws = nullptr;
     s.ws_bytes = 0;
+    if (s.tile_count) (void)hipFree(s.tile_count);
+    s.tile_count = nullptr;
     for (auto &p : s.free_events) {
         (void)hipEventDestroy(p.first);
         (void)hipEventDestroy(p.second);

@@ -21,10 +21,12 @@ RF_OK = 0
 
 
 class GemmConfig(ctypes.Structure):
-    _fields_ = [("variant", ctypes.c_int), ("split_k", ctypes.c_int), ("group_m", ctypes.c_int)]
+    _fields_ = [("variant", ctypes.c_int), ("split_k", ctypes.c_int), ("group_m", ctypes.c_int),
+                ("stream_k", ctypes.c_int)]
 
     def __repr__(self):
-        return "GemmConfig(variant=%d, split_k=%d, group_m=%d)" % (self.variant, self.split_k, self.group_m)
+        return "GemmConfig(variant=%d, split_k=%d, group_m=%d, stream_k=%d)" % (self.variant, self.split_k,
+                                                                                 self.group_m, self.stream_k)
 
 
 class PerfMetricEntry(ctypes.Structure):

@@ -31,7 +31,7 @@ def test_perf_metrics_layout_matches_the_reference_struct():
     assert ctypes.sizeof(PerfMetrics) == 4 + 20 * 28 == 564
     assert PerfMetrics.entries.offset == 4
     assert PerfMetricEntry.time.offset == 20 and PerfMetricEntry.gflops.offset == 24
-    assert ctypes.sizeof(GemmConfig) == 12
+    assert ctypes.sizeof(GemmConfig) == 16
 
 
 def test_status_codes_without_a_device():

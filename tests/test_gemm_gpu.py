@@ -59,7 +59,7 @@ def test_every_variant_and_split(rfk, gen, m, n, k):
         for split in (1, 2, 3):
             if split > k // 128:
                 continue
-            cfg = rfk.GemmConfig(v["variant"], split, 4)
+            cfg = rfk.GemmConfig(v["variant"], split, 4, 0)
             out = _run(rfk, data, config=cfg, canary=1024)
             assert_close_to_oracle(out, exp, RTOL, ATOL, "variant %r split %d" % (v, split))
             assert_few_mismatches_at_reference_atol(out, exp, "variant %r split %d" % (v, split))
@@ -78,11 +78,34 @@ def test_bit_exact_on_exactly_representable_data(rfk, m, n, k):
     tiled = m % 16 == 0 and n % 16 == 0
     plans = [None]
     if tiled:
-        plans += [rfk.GemmConfig(v["variant"], s, gm) for v in rfk.variants() for s, gm in ((1, 1), (2, 8), (3, 3))
+        plans += [rfk.GemmConfig(v["variant"], s, gm, 0) for v in rfk.variants() for s, gm in ((1, 1), (2, 8), (3, 3))
                   if s <= k // 128]
     for cfg in plans:
         out = _run(rfk, data, config=cfg, canary=1024)
         assert np.array_equal(bf16_bits(out), exp), "plan %r" % (cfg,)
+
+
+@pytest.mark.parametrize("m,n,k", [(2048, 2048, 512), (1536, 3072, 384), (4096, 4608, 1024), (6144, 4608, 256),
+                                   (1040, 2064, 640)])
+def test_stream_k_bit_exact_and_counters_self_reset(rfk, m, n, k):
+    """Persistent stream-K grid on shapes with at least as many tiles as CUs: equal shares of the work line cut
+    tiles at arbitrary K blocks, the last arriver sums the partials. Exact data makes any summation order give
+    the same bits. Run twice: the arrival counters must be back at zero after the first launch."""
+    data = exact_problem(m, n, k, seed=m + 3 * n + k)
+    exp = oracle_bf16(data)
+    ncu = torch.cuda.get_device_properties(0).multi_processor_count
+    tried = 0
+    for v in rfk.variants():
+        tiles = -(-m // v["block_m"]) * -(-n // v["block_n"])
+        if tiles < ncu:
+            continue
+        for gm in (1, 8):
+            cfg = rfk.GemmConfig(v["variant"], 1, gm, 1)
+            for rep in range(2):
+                out = _run(rfk, data, config=cfg, canary=1024)
+                assert np.array_equal(bf16_bits(out), exp), "plan %r rep %d" % (cfg, rep)
+            tried += 1
+    assert tried > 0
 
 
 @pytest.mark.parametrize("m,n,k", [(3, 130, 256), (1, 1, 128), (17, 64, 384), (5, 257, 128), (100, 72, 256)])
@@ -192,6 +215,6 @@ def test_status_codes(rfk):
     assert L.rf_fp8_gemm(p, p, p, p, p, 16, 16, 100, None) == 1      # RF_ERR_BAD_SHAPE
     assert L.rf_fp8_gemm(p, p, p, p, p, 0, 16, 128, None) == 1
     assert L.rf_fp8_gemm(None, p, p, p, p, 16, 16, 128, None) == 2   # RF_ERR_NULL_POINTER
-    bad = rfk.GemmConfig(99, 1, 1)
+    bad = rfk.GemmConfig(99, 1, 1, 0)
     assert L.rf_fp8_gemm_ex(p, p, p, p, p, 16, 16, 128, ctypes.byref(bad), None) == 4
     assert b"unsupported shape" in L.rf_gemm_last_error() or L.rf_gemm_last_error() != b""
