@@ -370,29 +370,51 @@ __device__ __forceinline__ void tile_mainloop(
 
 }
 
-// Stores a wave's accumulators: bf16 into C (masked at the M and N edges), or fp32 into a BM x BN workspace tile.
+// Stores a wave's accumulators as bf16 into C, masked at the M and N edges. In the MFMA layout a lane owns 4
+// consecutive n of one row, so a direct store instruction would touch 16 rows with 32-byte pieces. Instead each wave
+// stages its tile through its own LDS region (row = WN bf16 + 16 bytes of padding) and writes it back out with
+// 16 bytes per lane, 8 lanes per row: every store instruction covers whole 128-byte lines.
+// All waves must call it together: it starts with a barrier, because LDS-DMA loads of other waves may still be
+// landing in the stage buffers that are reused here.
 template <int BM, int BN, int WAVES_M, int WAVES_N>
 __device__ __forceinline__ void store_tile_bf16(const f32x4 (&acc)[BM / WAVES_M / 16][BN / WAVES_N / 16],
-                                                uint16_t *__restrict__ C, int M, int N, int m0, int n0) {
+                                                uint16_t *__restrict__ C, int M, int N, int m0, int n0, uint8_t *lds) {
     using G = TileGeom<BM, BN, WAVES_M, WAVES_N>;
+    constexpr int ROW = G::WN * 2 + 16;                  // bytes per staged row
+    constexpr int HALF_TM = G::TM / 2, ROWS = HALF_TM * 16;
+    constexpr int LPR = G::WN * 2 / 16;                  // lanes per row on the way out (16 bytes each)
+    constexpr int RPI = 64 / LPR;                        // rows per store instruction
+    static_assert(G::NW * ROWS * ROW <= 2 * G::STAGE, "staging fits in the stage buffers");
+    static_assert(ROWS % RPI == 0, "whole store instructions");
     // the opaque zero keeps this address arithmetic below the main loop: hoisted above it, it would cost the
     // loop dozens of registers
     int vz;
     asm volatile("v_mov_b32 %0, 0" : "=v"(vz));
     const int lane = (threadIdx.x & 63) + vz, wave = threadIdx.x >> 6, L = lane & 15, g = lane >> 4;
     const int wm = wave % WAVES_M, wn = wave / WAVES_M;
+    uint8_t *region = lds + wave * (ROWS * ROW);
+    __syncthreads();
 #pragma unroll
-    for (int j = 0; j < G::TM; j++) {
-        const int m = m0 + wm * G::WM + 16 * j + L;
+    for (int h = 0; h < 2; h++) {
 #pragma unroll
-        for (int i = 0; i < G::TN; i++) {
-            const int n = n0 + wn * G::WN + 16 * i + 4 * g;      // lane holds C[m][n..n+3]
-            if (m < M && n < N) {
+        for (int jj = 0; jj < HALF_TM; jj++) {
+            const int j = h * HALF_TM + jj;
+#pragma unroll
+            for (int i = 0; i < G::TN; i++) {            // lane holds C[16j + L][16i + 4g .. +3]
                 uint2 v;
                 v.x = pack_bf16x2(acc[j][i][0], acc[j][i][1]);
                 v.y = pack_bf16x2(acc[j][i][2], acc[j][i][3]);
-                *(uint2 *)(C + (size_t)m * N + n) = v;
+                *(uint2 *)(region + (16 * jj + L) * ROW + (16 * i + 4 * g) * 2) = v;
             }
+        }
+        // same wave writes and reads its region: program order is enough, the compiler inserts the LDS wait
+#pragma unroll
+        for (int r0 = 0; r0 < ROWS; r0 += RPI) {
+            const int r = r0 + lane / LPR, cb = (lane % LPR) * 16;          // row in the half, byte column
+            const uint4 v = *(const uint4 *)(region + r * ROW + cb);
+            const int m = m0 + wm * G::WM + h * ROWS + r;
+            const int n = n0 + wn * G::WN + cb / 2;
+            if (m < M && n < N) *(uint4 *)(C + (size_t)m * N + n) = v;
         }
     }
 }
@@ -451,7 +473,7 @@ __device__ __forceinline__ void exchange_tile_f32(f32x4 (&acc)[BM / WAVES_M / 16
 // One workgroup per (tile, K split). PARTIAL=false: writes bf16 C. PARTIAL=true: writes the fp32 partial sums of
 // the K range of split blockIdx.y to ws[split][M][N] (summed by reduce_splitk_bf16).
 // Requirements checked by the host: M%16==0, N%16==0, M>=16, N>=16, a/b 16-byte aligned,
-// c 8-byte aligned, K%128==0.
+// c 16-byte aligned, K%128==0.
 // ---------------------------------------------------------------------------------------------
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool PARTIAL>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_tile(
@@ -472,7 +494,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
         store_tile_f32<BM, BN, WAVES_M, WAVES_N>(acc, (float *)Cout + ((size_t)blockIdx.y * M + m0) * N + n0, N, M - m0,
                                                  N - n0);
     else
-        store_tile_bf16<BM, BN, WAVES_M, WAVES_N>(acc, (uint16_t *)Cout, M, N, m0, n0);
+        store_tile_bf16<BM, BN, WAVES_M, WAVES_N>(acc, (uint16_t *)Cout, M, N, m0, n0, lds);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -536,7 +558,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_str
                 write_c = true;
             }
         }
-        if (write_c) store_tile_bf16<BM, BN, WAVES_M, WAVES_N>(acc, C, M, N, m0, n0);
+        if (write_c) store_tile_bf16<BM, BN, WAVES_M, WAVES_N>(acc, C, M, N, m0, n0, lds);
         u = tq + kb1;
     }
 }

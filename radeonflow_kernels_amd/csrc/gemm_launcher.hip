@@ -115,7 +115,7 @@ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 bool tiled_path_ok(const void *a, const void *b, const void *c, int m, int n) {
     return m >= 16 && n >= 16 && m % 16 == 0 && n % 16 == 0 && ((uintptr_t)a % 16) == 0 && ((uintptr_t)b % 16) == 0 &&
-           ((uintptr_t)c % 8) == 0;
+           ((uintptr_t)c % 16) == 0;
 }
 
 // Plans measured on one MI355X by the tuner (python -m radeonflow_kernels_amd.tuner.gemm_tuner --all --emit).
