@@ -57,16 +57,30 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, h);
 }
 
-// Workgroup id -> (tile_m, tile_n). Workgroups are dealt round-robin to the 8 XCDs (each with its
-// own L2), so id%8 is the XCD. Give every XCD a contiguous range of logical tile ids, and order
-// logical ids in groups of `group_m` tile rows so that the tiles resident on one XCD at a time
-// form a compact patch that re-uses A rows and B columns from that XCD's L2.
+// Workgroup id -> (tile_m, tile_n). Workgroups are dealt round-robin to the 8 XCDs (each with its own L2), so
+// id%8 is the XCD. Whatever an XCD's workgroups read, its L2 has to fetch once: a band of full tile rows makes
+// every XCD read all of B. So, when the tile grid divides, the XCDs are laid out as a 4x2 (or 2x4, 8x1, 1x8) grid
+// of rectangular regions, as square as possible, and the workgroups of an XCD walk their region down the rows
+// first, so that the ~32 tiles in flight on the XCD form a compact patch sharing A rows and B columns. Otherwise
+// each XCD gets a contiguous range of tile ids, ordered in groups of `group_m` tile rows.
 __device__ __forceinline__ void tile_of_block(int bid, int nblocks, int tiles_m, int tiles_n, int group_m,
                                               bool xcd_remap, int &tile_m, int &tile_n) {
     int id = bid;
     if (xcd_remap) {
-        int xcd = bid % NUM_XCD, idx = bid / NUM_XCD;
-        int per = nblocks / NUM_XCD, rem = nblocks % NUM_XCD;
+        const int xcd = bid % NUM_XCD, idx = bid / NUM_XCD;
+        int xm = 0, xn = 0;                                   // XCD grid
+        if (tiles_m % 4 == 0 && tiles_n % 2 == 0 && tiles_m >= 2 * tiles_n / 2) { xm = 4; xn = 2; }
+        else if (tiles_m % 2 == 0 && tiles_n % 4 == 0) { xm = 2; xn = 4; }
+        else if (tiles_m % 4 == 0 && tiles_n % 2 == 0) { xm = 4; xn = 2; }
+        else if (tiles_m % 8 == 0) { xm = 8; xn = 1; }
+        else if (tiles_n % 8 == 0) { xm = 1; xn = 8; }
+        if (xm) {
+            const int rm = tiles_m / xm, rn = tiles_n / xn;   // region size in tiles; rm*rn workgroups per XCD
+            tile_m = (xcd % xm) * rm + idx % rm;
+            tile_n = (xcd / xm) * rn + idx / rm;
+            return;
+        }
+        const int per = nblocks / NUM_XCD, rem = nblocks % NUM_XCD;
         id = xcd * per + (xcd < rem ? xcd : rem) + idx;
     }
     int group_sz = group_m * tiles_n;
