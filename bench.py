@@ -108,6 +108,11 @@ def main():
     else:
         roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                     "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}
+    # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, scaled by a copy
+    # kernel (profiles/gemm_fp8_blockscale_tile_C2_hbm_traffic.txt); only known for the headline plan
+    if args.config == "C2" and (cfg.variant, cfg.split_k, cfg.stream_k) == (0, 1, 0):
+        roofline["traffic"] = 385.4e6
+        roofline["traffic_note"] = "fetch 328.8 MB + write 56.6 MB per launch, profiles/gemm_fp8_blockscale_tile_C2_hbm_traffic.txt"
     roofline["kernel"] = "gemm_fp8_blockscale_tile (variant %d, split_k %d)" % (cfg.variant, cfg.split_k)
     roofline["avg_launch_us"] = round(us, 2)
     roofline["algorithmic_flop_per_launch"] = flop
@@ -123,7 +128,7 @@ def main():
         "data": "synthetic (seeded N(0,1) fp32 -> e4m3fn, amax/448 block scales), random inputs resident in HBM",
         "config": {"workload": "%s: blockscaled fp8 GEMM M=%d N=%d K=%d, a[K][M] b[K][N] fp8, fp32 scales, bf16 C"
                                % (args.config, m, n, k),
-                   "plan": {"variant": cfg.variant, "split_k": cfg.split_k, "group_m": cfg.group_m},
+                   "plan": {"variant": cfg.variant, "split_k": cfg.split_k, "group_m": cfg.group_m, "stream_k": cfg.stream_k},
                    "device": prop.name, "compute_units": prop.multi_processor_count, "clock_mhz": clock_mhz,
                    "derived_fp8_peak_tflops": round(derived_peak, 1), "input_generation_s": round(gen_s, 2)},
         "roofline": roofline,
