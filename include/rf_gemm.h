@@ -73,6 +73,8 @@ int rf_gemm_select_config(int m, int n, int k, rf_gemm_config *out);
 /* Variant table introspection (for the tuner and tests). Returns RF_ERR_BAD_CONFIG past the end. */
 int rf_gemm_num_variants(void);
 int rf_gemm_variant_info(int variant, int *block_m, int *block_n, int *waves_m, int *waves_n, int *lds_bytes);
+/* 1 if the variant can run with rf_gemm_config.stream_k = 1, 0 if not (or if the index is out of range). */
+int rf_gemm_variant_has_stream_k(int variant);
 
 /* Device workspace (split-K partial sums) needed for a shape under the automatic plan, in bytes. */
 size_t rf_gemm_workspace_bytes(int m, int n, int k);

@@ -43,11 +43,19 @@ constexpr int NUM_XCD = 8;
 
 // XOR applied to the 16-byte-chunk index of LDS row k (row width W bytes). Chosen so that the 32
 // lanes the LDS serves together in a transpose read (two 16-lane groups: 8 k-rows x 2 half-chunks
-// each, the groups 32 rows apart) touch all 64 banks exactly once.
+// each, the groups 32 rows apart) touch all 64 banks exactly once. Row k starts W/16 * k chunks into
+// the 16-chunk bank period; with W/16 = 2^e * odd, rows 2^(4-e) apart (and rows 32 apart) start on
+// the same chunk, and the XOR spreads exactly those over the low e bits of the chunk index. It never
+// leaves an aligned group of 2^e chunks, so it also works for rows of 12, 14 or 18 chunks.
+template <int W>
+constexpr int swizzle_bits() {
+    static_assert(W % 32 == 0, "tile row width");
+    constexpr int q = W / 16;
+    return (q % 16 == 0) ? 4 : (q % 8 == 0) ? 3 : (q % 4 == 0) ? 2 : 1;
+}
 template <int W>
 __device__ __forceinline__ int swizzle_of_row(int k) {
-    constexpr int r = (W == 256) ? 0 : (W == 128) ? 1 : 2;   // log2(rows per 256 B bank wrap)
-    static_assert(W == 256 || W == 128 || W == 64, "tile row width");
+    constexpr int r = 4 - swizzle_bits<W>();                 // log2(rows per bank period)
     return ((k & 7) >> r) | (((k >> 5) & 1) << (3 - r));
 }
 

@@ -15,6 +15,7 @@
 
 #include "../../include/rf_gemm.h"
 #include "fp8_gemm_kernels.h"
+#include "fp8_gemm_hold_a.h"
 
 namespace {
 
@@ -37,22 +38,29 @@ typedef void (*tile_kernel_t)(const uint8_t *, const uint8_t *, const float *, c
 typedef void (*streamk_kernel_t)(const uint8_t *, const uint8_t *, const float *, const float *, uint16_t *, int, int,
                                  int, int, int, int, unsigned *, float *);
 struct Variant {
-    int bm, bn, waves_m, waves_n;
+    int bm, bn, waves_m, waves_n, lds;
     tile_kernel_t direct, partial;
-    streamk_kernel_t streamk;
-    int lds_bytes() const { return 2 * (rf::BK * (bm + bn) + 4 * bm) + 16; }
+    streamk_kernel_t streamk;            // null: the variant has no stream-K form
+    int lds_bytes() const { return lds; }
     int threads() const { return waves_m * waves_n * 64; }
 };
 #define RF_VARIANT(BM, BN, WM, WN)                                                         \
-    Variant { BM, BN, WM, WN, rf::gemm_fp8_blockscale_tile<BM, BN, WM, WN, false>,         \
+    Variant { BM, BN, WM, WN, rf::TileGeom<BM, BN, WM, WN>::LDS_BYTES,                     \
+              rf::gemm_fp8_blockscale_tile<BM, BN, WM, WN, false>,                         \
               rf::gemm_fp8_blockscale_tile<BM, BN, WM, WN, true>,                          \
               rf::gemm_fp8_blockscale_streamk<BM, BN, WM, WN> }
+// tiles with sides that are not powers of two (A fragments held, B streamed)
+#define RF_VARIANT_HOLD_A(BM, BN, WM, WN)                                                  \
+    Variant { BM, BN, WM, WN, rf::HoldAGeom<BM, BN, WM, WN>::LDS_BYTES,                    \
+              rf::gemm_fp8_blockscale_tile_hold_a<BM, BN, WM, WN, false>,                  \
+              rf::gemm_fp8_blockscale_tile_hold_a<BM, BN, WM, WN, true>, nullptr }
 const Variant kVariants[] = {
     RF_VARIANT(256, 256, 2, 4),   // 0: 8 waves, wave tile 128(m) x 64(n), 128 KiB LDS
     RF_VARIANT(128, 128, 2, 2),   // 1: 4 waves, wave tile 64 x 64, 64 KiB LDS (2 workgroups per CU)
     RF_VARIANT(256, 128, 2, 2),   // 2: 4 waves, wave tile 128 x 64, 96 KiB LDS
     RF_VARIANT(128, 256, 2, 4),   // 3: 8 waves, wave tile 64 x 64, 96 KiB LDS
     RF_VARIANT(128, 64, 2, 1),    // 4: 2 waves, wave tile 64 x 64, 48 KiB LDS (3 workgroups per CU)
+    RF_VARIANT_HOLD_A(192, 288, 4, 2),   // 5: 8 waves, wave tile 48 x 144, 122 KiB LDS (6144 x 4608 = 512 tiles)
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
@@ -83,7 +91,8 @@ int ensure_device_info(State &s) {
     for (const Variant &v : kVariants) {
         RF_HIP(hipFuncSetAttribute((const void *)v.direct, hipFuncAttributeMaxDynamicSharedMemorySize, v.lds_bytes()));
         RF_HIP(hipFuncSetAttribute((const void *)v.partial, hipFuncAttributeMaxDynamicSharedMemorySize, v.lds_bytes()));
-        RF_HIP(hipFuncSetAttribute((const void *)v.streamk, hipFuncAttributeMaxDynamicSharedMemorySize, v.lds_bytes()));
+        if (v.streamk)
+            RF_HIP(hipFuncSetAttribute((const void *)v.streamk, hipFuncAttributeMaxDynamicSharedMemorySize, v.lds_bytes()));
     }
     s.attrs_set = true;
     return RF_OK;
@@ -188,6 +197,7 @@ int launch(const void *a, const void *b, const float *as, const float *bs, void 
             return fail(RF_ERR_BAD_CONFIG, "configuration not usable for this shape");
         if (cfg.stream_k != 0) {
             const Variant &sv = kVariants[cfg.variant];
+            if (!sv.streamk) return fail(RF_ERR_BAD_CONFIG, "this variant has no stream_k form");
             const long t = (long)ceil_div(m, sv.bm) * ceil_div(n, sv.bn);
             if (t < s.num_cu || t > kMaxStreamKTiles)
                 return fail(RF_ERR_BAD_CONFIG, "stream_k needs at least as many tiles as compute units");
@@ -300,6 +310,10 @@ int rf_gemm_variant_info(int variant, int *block_m, int *block_n, int *waves_m, 
     if (waves_n) *waves_n = v.waves_n;
     if (lds_bytes) *lds_bytes = v.lds_bytes();
     return RF_OK;
+}
+
+int rf_gemm_variant_has_stream_k(int variant) {
+    return variant >= 0 && variant < kNumVariants && kVariants[variant].streamk != nullptr;
 }
 
 size_t rf_gemm_workspace_bytes(int m, int n, int k) {
