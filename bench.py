@@ -226,6 +226,28 @@ def main():
                 par["mismatches"] if par else "-", par["mismatches_at_reference_atol_1e-3"] if par else "-",
                 par[err_key[0]] if par else "-", rfk.select_config(mm, nn, kk)), file=sys.stderr)
             del gg, dd
+        # the block quantisers that produce the operands (HBM-bound: source read once, fp8 + scales written once)
+        out["quantisers"] = {}
+        for label, fn, rows in (("quantize_a", rfk.quantize_a, m), ("quantize_b", rfk.quantize_b, n)):
+            for dt in (torch.float32, torch.bfloat16):
+                src = torch.randn((rows, k), device="cuda", dtype=dt)
+                with torch.cuda.stream(stream):
+                    for _ in range(10):
+                        fn(src)
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record(stream)
+                    for _ in range(20):
+                        fn(src)
+                    e1.record(stream)
+                    stream.synchronize()
+                u = e0.elapsed_time(e1) * 1e3 / 20
+                nbytes = rows * k * (src.element_size() + 1) + 4 * (k // 128) * (rows if label == "quantize_a" else (rows + 127) // 128)
+                key = "%s_%s_%dx%d" % (label, "f32" if dt == torch.float32 else "bf16", rows, k)
+                out["quantisers"][key] = {"us": round(u, 2), "gbs": round(nbytes / u / 1e3, 1),
+                                          "pct_hbm_peak": round(100 * nbytes / u / 1e3 / PEAK_HBM_GBS, 2)}
+                print("%-34s %8.2f us %8.1f GB/s (%.1f %% of 8 TB/s; includes the allocation of the outputs by torch)"
+                      % (key, u, nbytes / u / 1e3, 100 * nbytes / u / 1e3 / PEAK_HBM_GBS), file=sys.stderr)
+                del src
     print(json.dumps(out))
     return 0
 

@@ -85,6 +85,19 @@ size_t rf_gemm_workspace_bytes(int m, int n, int k);
 int rf_gemm_init(size_t workspace_bytes);
 void rf_gemm_destroy(void);
 
+/* Block quantisers: the step before the GEMM, on the GPU. No counterpart in the reference, whose harness draws
+ * fp8 bytes and scales directly (tests/gemm/gemm_test.cpp:64-99); they implement the recipe its callers use:
+ * scale = amax/448 over a block (1 if the block is all zero), value = e4m3fn_rne(x / scale).
+ *   rf_quantize_a_*: x is [m][k] row-major (fp32 or bf16), one scale per (row, 128-wide K block);
+ *                    writes a ([K][M] fp8, the layout `run` takes) and as ([K/128][M] fp32).
+ *   rf_quantize_b_*: w is [n][k] row-major, one scale per 128x128 block (the last N block may be partial);
+ *                    writes b ([K][N] fp8) and bs ([K/128][ceil(N/128)] fp32).
+ * k must be a positive multiple of 128; sources 16-byte aligned (bf16: 8). Enqueued on `stream`. */
+int rf_quantize_a_f32(const float *x, int m, int k, void *a, float *as, hipStream_t stream);
+int rf_quantize_a_bf16(const void *x, int m, int k, void *a, float *as, hipStream_t stream);
+int rf_quantize_b_f32(const float *w, int n, int k, void *b, float *bs, hipStream_t stream);
+int rf_quantize_b_bf16(const void *w, int n, int k, void *b, float *bs, hipStream_t stream);
+
 /* Text of the last failure on this thread's most recent rf_* call ("" if none). */
 const char *rf_gemm_last_error(void);
 

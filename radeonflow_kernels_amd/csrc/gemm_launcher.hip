@@ -16,6 +16,7 @@
 #include "../../include/rf_gemm.h"
 #include "fp8_gemm_kernels.h"
 #include "fp8_gemm_hold_a.h"
+#include "quantize_kernels.h"
 
 namespace {
 
@@ -357,6 +358,50 @@ void rf_gemm_destroy(void) {
 }
 
 const char *rf_gemm_last_error(void) { return g_last_error.c_str(); }
+
+}  // extern "C"
+
+namespace {
+// rows x K source (row-major, K contiguous) -> fp8 [K][rows] + scales; see quantize_kernels.h
+template <bool PER_ROW, bool IN_BF16>
+int launch_quantize(const void *x, int rows, int k, void *out, float *scales, hipStream_t stream) {
+    g_last_error.clear();
+    if (rows < 1 || k < rf::BK || k % rf::BK != 0)
+        return fail(RF_ERR_BAD_SHAPE, "unsupported shape rows=" + std::to_string(rows) + " K=" + std::to_string(k) +
+                                          " (need rows>=1, K a positive multiple of 128)");
+    if (!x || !out || !scales) return fail(RF_ERR_NULL_POINTER, "null device pointer");
+    if ((uintptr_t)x % (IN_BF16 ? 8 : 16) != 0 || (uintptr_t)scales % 4 != 0)
+        return fail(RF_ERR_BAD_CONFIG, "source must be 16-byte aligned (8 for bf16), scales 4-byte aligned");
+    State &s = state();
+    {
+        std::lock_guard<std::mutex> lock(s.mu);
+        int rc = ensure_device_info(s);
+        if (rc != RF_OK) return rc;
+    }
+    const bool vector_store = rows % 16 == 0 && (uintptr_t)out % 16 == 0;
+    const int row_blocks = ceil_div(rows, 128);
+    dim3 grid(row_blocks, k / rf::BK);
+    hipLaunchKernelGGL((rf::quantize_block128<PER_ROW, IN_BF16>), grid, dim3(256), 0, stream, x, rows, k, (uint8_t *)out,
+                       scales, PER_ROW ? rows : row_blocks, vector_store);
+    RF_HIP(hipGetLastError());
+    return RF_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int rf_quantize_a_f32(const float *x, int m, int k, void *a, float *as, hipStream_t stream) {
+    return launch_quantize<true, false>(x, m, k, a, as, stream);
+}
+int rf_quantize_a_bf16(const void *x, int m, int k, void *a, float *as, hipStream_t stream) {
+    return launch_quantize<true, true>(x, m, k, a, as, stream);
+}
+int rf_quantize_b_f32(const float *w, int n, int k, void *b, float *bs, hipStream_t stream) {
+    return launch_quantize<false, false>(w, n, k, b, bs, stream);
+}
+int rf_quantize_b_bf16(const void *w, int n, int k, void *b, float *bs, hipStream_t stream) {
+    return launch_quantize<false, true>(w, n, k, b, bs, stream);
+}
 
 void run(void *a, void *b, void *as, void *bs, void *c, int m, int n, int k, PerfMetrics *metrics,
          hipStream_t job_stream0) {

@@ -39,7 +39,7 @@ class PerfMetrics(ctypes.Structure):
 
 EXPORTS = ("run", "rf_fp8_gemm", "rf_fp8_gemm_ex", "rf_gemm_select_config", "rf_gemm_num_variants",
            "rf_gemm_variant_info", "rf_gemm_variant_has_stream_k", "rf_gemm_workspace_bytes", "rf_gemm_init", "rf_gemm_destroy",
-           "rf_gemm_last_error")
+           "rf_gemm_last_error", "rf_quantize_a_f32", "rf_quantize_a_bf16", "rf_quantize_b_f32", "rf_quantize_b_bf16")
 
 
 def lib():
@@ -70,6 +70,10 @@ def lib():
         L.rf_gemm_init.restype = i32
         L.rf_gemm_destroy.restype = None
         L.rf_gemm_last_error.restype = ctypes.c_char_p
+        for name in ("rf_quantize_a_f32", "rf_quantize_a_bf16", "rf_quantize_b_f32", "rf_quantize_b_bf16"):
+            f = getattr(L, name)
+            f.argtypes = [ctypes.c_void_p, i32, i32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+            f.restype = i32
         _lib = L
     return _lib
 
@@ -129,6 +133,35 @@ def run_with_metrics(a, b, a_scale, b_scale, c):
                   ctypes.byref(pm), stream)
         torch.cuda.synchronize(a.device)
     return pm.entries[0].time, pm.entries[0].gflops, pm.count
+
+
+def _quantize(x, per_row):
+    if x.dim() != 2 or not x.is_contiguous() or x.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("source must be a contiguous 2-D fp32 or bf16 tensor [rows, K]")
+    rows, k = x.shape
+    if k < 128 or k % 128:
+        raise ValueError("K must be a positive multiple of 128")
+    q = torch.empty((k, rows), dtype=torch.float8_e4m3fn, device=x.device)
+    nscale = rows if per_row else (rows + 127) // 128
+    scales = torch.empty((k // 128, nscale), dtype=torch.float32, device=x.device)
+    name = "rf_quantize_%s_%s" % ("a" if per_row else "b", "f32" if x.dtype == torch.float32 else "bf16")
+    stream = ctypes.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)
+    with torch.cuda.device(x.device):
+        rc = getattr(lib(), name)(x.data_ptr(), rows, k, q.data_ptr(), scales.data_ptr(), stream)
+    if rc != RF_OK:
+        raise RuntimeError("%s failed (%d): %s" % (name, rc, last_error()))
+    return q.T, scales.T         # the transposed views fp8_mm takes: [rows, K] stride (1, rows), [rows or QN, K/128]
+
+
+def quantize_a(x):
+    """Activations [M, K] (fp32 or bf16, on the GPU) -> (a, a_scale) as fp8_mm takes them: one scale per
+    (row, 128-wide K block), scale = amax/448, value = e4m3fn_rne(x / scale)."""
+    return _quantize(x, True)
+
+
+def quantize_b(w):
+    """Weights [N, K] -> (b, b_scale): one scale per 128x128 block."""
+    return _quantize(w, False)
 
 
 def select_config(m, n, k):

@@ -1,0 +1,106 @@
+"""GPU block quantisers against the CPU oracle's quantisers: bytes and scales must agree bit for bit
+(integer / byte work; the only float steps are two correctly rounded fp32 divisions)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import cref, ref_kernel as rk
+from helpers import RTOL, ATOL, assert_close_to_oracle, oracle_bf16
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def rfk():
+    import radeonflow_kernels_amd as m
+    m.lib()
+    return m
+
+
+def _source(rows, k, seed, kind):
+    x = cref.randn(seed, rows * k).reshape(rows, k)
+    if kind == "wide":          # many binades, exact zeros, negative zeros, a zero block, a huge value
+        x = x * np.exp2(np.floor(cref.randn(seed + 1, rows * k).reshape(rows, k) * 6)).astype(np.float32)
+        x[::7, ::5] = 0.0
+        x[1::11, 3::13] = -0.0
+        x[: min(rows, 3), :128] = 0.0
+        x[rows // 2, k // 2] = 3.0e38
+        x[rows - 1, k - 1] = 1.0e-41        # fp32 denormal
+    return np.ascontiguousarray(x, dtype=np.float32)
+
+
+def _unpack(q, s):
+    """(fp8 view [rows,K] stride (1,rows), scales view) -> numpy arrays in the launcher's memory layouts."""
+    return q.T.contiguous().view(torch.uint8).cpu().numpy(), s.T.contiguous().cpu().numpy()
+
+
+@pytest.mark.parametrize("kind", ["normal", "wide"])
+@pytest.mark.parametrize("rows,k", [(128, 128), (256, 512), (1024, 7168), (576, 1024), (200, 256), (1, 128), (33, 384),
+                                    (6144, 256)])
+def test_quantize_a_matches_oracle_bit_for_bit(rfk, rows, k, kind):
+    x = _source(rows, k, 1000 + rows + k, kind)
+    a_ref, as_ref = cref.quantize_a(x)
+    q, s = rfk.quantize_a(torch.from_numpy(x).cuda())
+    torch.cuda.synchronize()
+    assert q.shape == (rows, k) and q.stride() == (1, rows) and s.shape == (rows, k // 128)
+    a_gpu, as_gpu = _unpack(q, s)
+    assert np.array_equal(as_gpu.view(np.uint32), np.asarray(as_ref).view(np.uint32))
+    assert np.array_equal(a_gpu, np.asarray(a_ref))
+
+
+@pytest.mark.parametrize("kind", ["normal", "wide"])
+@pytest.mark.parametrize("rows,k", [(128, 128), (256, 512), (1536, 7168), (576, 1024), (200, 256), (1, 128), (33, 384)])
+def test_quantize_b_matches_oracle_bit_for_bit(rfk, rows, k, kind):
+    w = _source(rows, k, 2000 + rows + k, kind)
+    b_ref, bs_ref = cref.quantize_b(w)
+    q, s = rfk.quantize_b(torch.from_numpy(w).cuda())
+    torch.cuda.synchronize()
+    assert s.shape == ((rows + 127) // 128, k // 128)
+    b_gpu, bs_gpu = _unpack(q, s)
+    assert np.array_equal(bs_gpu.view(np.uint32), np.asarray(bs_ref).view(np.uint32))
+    assert np.array_equal(b_gpu, np.asarray(b_ref))
+
+
+@pytest.mark.parametrize("rows,k", [(256, 512), (200, 256)])
+def test_bf16_sources_equal_fp32_sources_of_the_same_values(rfk, rows, k):
+    x = torch.from_numpy(_source(rows, k, 77, "normal")).bfloat16()
+    qa, sa = rfk.quantize_a(x.cuda())
+    qa32, sa32 = rfk.quantize_a(x.float().cuda())
+    qb, sb = rfk.quantize_b(x.cuda())
+    qb32, sb32 = rfk.quantize_b(x.float().cuda())
+    torch.cuda.synchronize()
+    for got, exp in ((qa, qa32), (qb, qb32)):
+        assert torch.equal(got.view(torch.uint8), exp.view(torch.uint8))
+    assert torch.equal(sa, sa32) and torch.equal(sb, sb32)
+
+
+def test_quantise_then_gemm_end_to_end(rfk):
+    """fp32 activations and weights quantised on the GPU and multiplied on the GPU, against the oracle GEMM run on
+    the oracle's own quantisation of the same sources."""
+    m, n, k = 512, 576, 1024
+    x = cref.randn(4242, m * k).reshape(m, k)
+    w = cref.randn(4243, n * k).reshape(n, k)
+    qa, sa = rfk.quantize_a(torch.from_numpy(x).cuda())
+    qb, sb = rfk.quantize_b(torch.from_numpy(w).cuda())
+    out = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda:0")
+    rfk.fp8_mm(qa, qb, sa, sb, out)
+    torch.cuda.synchronize()
+    a_ref, as_ref = cref.quantize_a(x)
+    b_ref, bs_ref = cref.quantize_b(w)
+
+    def views(codes, scales):          # [K][rows] storage -> the [rows, K] views ref_kernel takes
+        return torch.from_numpy(np.asarray(codes)).view(torch.float8_e4m3fn).T, torch.from_numpy(np.asarray(scales)).T
+    a_t, as_t = views(a_ref, as_ref)
+    b_t, bs_t = views(b_ref, bs_ref)
+    exp = oracle_bf16((a_t, b_t, as_t, bs_t, torch.zeros((m, n), dtype=torch.bfloat16)))
+    assert_close_to_oracle(out, exp, RTOL, ATOL, "quantise + gemm")
+
+
+def test_status_codes(rfk):
+    L = rfk.lib()
+    x = torch.zeros((128, 128), device="cuda")
+    q = torch.empty((128, 128), dtype=torch.uint8, device="cuda")
+    s = torch.empty((1, 128), device="cuda")
+    assert L.rf_quantize_a_f32(x.data_ptr(), 128, 100, q.data_ptr(), s.data_ptr(), None) == 1     # RF_ERR_BAD_SHAPE
+    assert L.rf_quantize_a_f32(None, 128, 128, q.data_ptr(), s.data_ptr(), None) == 2            # RF_ERR_NULL_POINTER
+    assert L.rf_quantize_a_f32(x.data_ptr() + 4, 127, 128, q.data_ptr(), s.data_ptr(), None) == 4  # misaligned source
