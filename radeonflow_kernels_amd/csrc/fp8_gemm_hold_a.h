@@ -165,11 +165,13 @@ __device__ __forceinline__ void tile_mainloop_hold_a(
 
     i32x8 afrag[TM], bfrag[NBUF];
     f32x4 pring[PR];
-    float s0[TM], s1[TM], sprev[TM], sraw[4], sb0_cur = 0.f, sb1_cur = 0.f, sb0_next = 0.f, sb1_next = 0.f;
+    // sc: the scales the folds use right now (sa*sb of the b_scale block the current n-tile row lies in); s1: the
+    // scales of the wave's second b_scale block, swapped in when the folds reach n-tile ib
+    float sc[TM], s1[TM], sraw[4], sb0_cur = 0.f, sb1_cur = 0.f, sb0_next = 0.f, sb1_next = 0.f;
 #pragma unroll
     for (int r = 0; r < PR; r++) pring[r] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int j = 0; j < TM; j++) s0[j] = s1[j] = sprev[j] = 0.f;
+    for (int j = 0; j < TM; j++) sc[j] = s1[j] = 0.f;
 
     auto rd = [&](uint32_t off) { return __builtin_amdgcn_ds_read_tr8_b64_v2i32((RF_LDS i32x2 *)(lds + off)); };
     auto read_b_part = [&](int buf, int i, uint32_t stage_base, int t) {
@@ -216,12 +218,6 @@ __device__ __forceinline__ void tile_mainloop_hold_a(
         const int kn1 = clamp_kb(kb + 1), kn2 = clamp_kb(kb + 2);
         const uint8_t *a1 = src_a_of(kn1), *b1 = src_b_of(kn1), *q1 = src_s_of(kn1);
         const uint8_t *a2 = src_a_of(kn2), *b2 = src_b_of(kn2), *q2 = src_s_of(kn2);
-#pragma unroll
-        for (int j = 0; j < TM; j++) {
-            sprev[j] = (TN - 1 < ib) ? s0[j] : s1[j];      // scales of the previous block's last n-tile (lagged folds)
-            s0[j] = sraw[j] * sb0_cur;
-            s1[j] = sraw[j] * sb1_cur;
-        }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int t = 0; t < NMFMA; t++) {
@@ -257,13 +253,28 @@ __device__ __forceinline__ void tile_mainloop_hold_a(
                 read_a(j, nxt);                                    // afrag[j] is dead: refill for block kb+1
                 if (j == 0) read_scales(nxt);
             }
-            // lagged fold
+            // lagged fold. The first LAG slots fold the tail of the previous K block with the scales it left in
+            // sc; when the folds reach n-tile 0 of this block sc is recomputed, when they reach n-tile ib (if the
+            // wave has a second b_scale block) s1 is swapped in: a wave-uniform branch around TM moves.
             {
-                const bool tail = t < LAG;                         // folds owed by the previous K block
+                const bool tail = t < LAG;
                 const int u = tail ? NMFMA + t - LAG : t - LAG, iu = u / TM, ju = u % TM;
-                const float sc = tail ? sprev[ju] : iu == 0 ? s0[ju] : (iu < ib) ? s0[ju] : s1[ju];
+                if (!tail && ju == 0) {
+                    if (iu == 0) {
 #pragma unroll
-                for (int e = 0; e < 4; e++) acc[ju][iu][e] = __builtin_fmaf(sc, pring[u % PR][e], acc[ju][iu][e]);
+                        for (int j2 = 0; j2 < TM; j2++) {
+                            sc[j2] = sraw[j2] * sb0_cur;
+                            s1[j2] = sraw[j2] * sb1_cur;
+                        }
+                    } else if (iu == ib) {
+                        // moves written as asm so that they stay behind a scalar branch (taken once per K block)
+                        // instead of becoming TM selects in every n-tile row
+#pragma unroll
+                        for (int j2 = 0; j2 < TM; j2++) asm volatile("v_mov_b32 %0, %1" : "+v"(sc[j2]) : "v"(s1[j2]));
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[ju][iu][e] = __builtin_fmaf(sc[ju], pring[u % PR][e], acc[ju][iu][e]);
                 asm volatile("" : "+v"(acc[ju][iu]));        // anchor: the fold happens in this slot
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -275,9 +286,8 @@ __device__ __forceinline__ void tile_mainloop_hold_a(
 #pragma unroll
     for (int t = 0; t < LAG; t++) {
         const int u = NMFMA + t - LAG, iu = u / TM, ju = u % TM;
-        const float sc = (iu < ib) ? s0[ju] : s1[ju];
 #pragma unroll
-        for (int e = 0; e < 4; e++) acc[ju][iu][e] = __builtin_fmaf(sc, pring[u % PR][e], acc[ju][iu][e]);
+        for (int e = 0; e < 4; e++) acc[ju][iu][e] = __builtin_fmaf(sc[ju], pring[u % PR][e], acc[ju][iu][e]);
     }
     // LDS-DMA writes of the last (redundant) prefetches must land before this workgroup's LDS can be handed on
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");

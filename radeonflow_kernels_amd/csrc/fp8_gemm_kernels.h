@@ -36,6 +36,7 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int BK = 128;        // K per stage == the quantisation block
+template <int V> struct IntTag { static constexpr int value = V; };
 constexpr int NUM_XCD = 8;
 
 #define RF_LDS __attribute__((address_space(3)))
@@ -121,8 +122,13 @@ __device__ __forceinline__ void tile_mainloop(
     constexpr int NW = WAVES_M * WAVES_N;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     constexpr int TM = WM / 16, TN = WN / 16;
-    // one LDS stage: A[128][BM] bytes, B[128][BN] bytes, then BM fp32 a_scale values
+    // one LDS stage: A[128][BM] bytes, B[128][BN] bytes and BM fp32 a_scale values. The two stages are interleaved
+    // by operand (A0 A1 B0 B1 S0 S1), so that a transpose read of either stage is "per-lane base register + a
+    // 16-bit immediate": no address arithmetic in the loop.
     constexpr int STAGE_A = BK * BM, STAGE_B = BK * BN, STAGE_S = BM * 4, STAGE = STAGE_A + STAGE_B + STAGE_S;
+    constexpr int OFF_B = 2 * STAGE_A, OFF_S = 2 * STAGE_A + 2 * STAGE_B;
+    static_assert(STAGE_A + 3 * 8 * BM + 16 * (BM / 16) < 65536 && STAGE_B + 3 * 8 * BN + 16 * (BN / 16) < 65536,
+                  "stage offsets must fit the immediate offset of an LDS read");
     constexpr int INST_A = STAGE_A / 1024 / NW, INST_B = STAGE_B / 1024 / NW;   // 1 KiB per wave instruction
     constexpr int NSC = BM / 64;                                                // scale loads: 64 floats each
     static_assert(STAGE_A % (1024 * NW) == 0 && STAGE_B % (1024 * NW) == 0, "loads must divide evenly over waves");
@@ -192,8 +198,8 @@ __device__ __forceinline__ void tile_mainloop(
     // DMA instruction d of this wave: A rows (d < INST_A), then B rows, then the scales. Its global source for K
     // block kb is dma_src(d, kb); its LDS destination inside a stage is fixed. In the loop each instruction keeps a
     // running source pointer (one 64-bit scalar add per K block) instead of recomputing products.
-    const uint32_t lds_dst_a = lds_base + wave * (INST_A * 1024), lds_dst_b = lds_base + STAGE_A + wave * (INST_B * 1024),
-                   lds_dst_s = lds_base + STAGE_A + STAGE_B + wave * 256;
+    const uint32_t lds_dst_a = lds_base + wave * (INST_A * 1024), lds_dst_b = lds_base + OFF_B + wave * (INST_B * 1024),
+                   lds_dst_s = lds_base + OFF_S + wave * 256;
     auto dma_src = [&](int d, int kb) -> const uint8_t * {
         if (d < INST_A) return A + ((size_t)kb * BK + (size_t)(wave * INST_A + d) * RPI_A) * M;
         if (d < INST_A + INST_B) return B + ((size_t)kb * BK + (size_t)(wave * INST_B + (d - INST_A)) * RPI_B) * N;
@@ -202,19 +208,19 @@ __device__ __forceinline__ void tile_mainloop(
     auto dma_step = [&](int d) -> size_t {       // bytes from one K block to the next
         return d < INST_A ? (size_t)BK * M : d < INST_A + INST_B ? (size_t)BK * N : (size_t)M * 4;
     };
-    auto issue_dma = [&](int d, uint32_t stage_off, const uint8_t *src) {
+    auto issue_dma = [&](int d, int stage, const uint8_t *src) {
         if (d < INST_A) {
             asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                         :: "v"(goff_a[cls_a(d < INST_A ? d : 0)]), "s"(src), "s"(stage_off + lds_dst_a), "n"(d * 1024)
+                         :: "v"(goff_a[cls_a(d < INST_A ? d : 0)]), "s"(src), "s"(lds_dst_a), "n"(d * 1024 + stage * STAGE_A)
                          : "memory", "scc");
         } else if (d < INST_A + INST_B) {
             const int e = d - INST_A < INST_B ? d - INST_A : 0;
             asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                         :: "v"(goff_b[cls_b(e >= 0 ? e : 0)]), "s"(src), "s"(stage_off + lds_dst_b), "n"(e * 1024)
+                         :: "v"(goff_b[cls_b(e >= 0 ? e : 0)]), "s"(src), "s"(lds_dst_b), "n"(e * 1024 + stage * STAGE_B)
                          : "memory", "scc");
         } else if (wave < NSC) {
-            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
-                         :: "v"(goff_s), "s"(src), "s"(stage_off + lds_dst_s) : "memory");
+            asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+                         :: "v"(goff_s), "s"(src), "s"(lds_dst_s), "n"(stage * STAGE_S) : "memory", "scc");
         }
     };
 
@@ -225,8 +231,9 @@ __device__ __forceinline__ void tile_mainloop(
     // (TM, TN powers of two): one base register per operand, the tile index is XORed in at the use.
     static_assert((TM & (TM - 1)) == 0 && (TN & (TN - 1)) == 0, "tile counts are powers of two");
     const uint32_t aoff_base = krow * BM + (((wm * TM) ^ swizzle_of_row<BM>(krow)) << 4) + 8 * (L & 1);
-    const uint32_t boff_base = krow * BN + (((wn * TN) ^ swizzle_of_row<BN>(krow)) << 4) + 8 * (L & 1);
-    const uint32_t soff = STAGE_A + STAGE_B + (wm * WM + L * TM) * 4;   // this lane's TM scales
+    // (OFF_B has no low bits set, so it passes through the XOR with the tile index unchanged)
+    const uint32_t boff_base = OFF_B + krow * BN + (((wn * TN) ^ swizzle_of_row<BN>(krow)) << 4) + 8 * (L & 1);
+    const uint32_t soff = OFF_S + (wm * WM + L * TM) * 4;               // this lane's TM scales
 
     int nb = (n0 + wn * WN) >> 7;
     if (nb > QN - 1) nb = QN - 1;
@@ -271,26 +278,26 @@ __device__ __forceinline__ void tile_mainloop(
     auto rd = [&](uint32_t stage_base, uint32_t off) {
         return __builtin_amdgcn_ds_read_tr8_b64_v2i32((RF_LDS i32x2 *)(lds + stage_base + off));
     };
-    auto read_bfrag = [&](int i, uint32_t stage_base) {
+    auto read_bfrag = [&](int i, int stage) {
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-            i32x2 v = rd(stage_base, (boff_base ^ (i << 4)) + STAGE_A + t * 8 * BN);
+            i32x2 v = rd(stage * STAGE_B, (boff_base ^ (i << 4)) + t * 8 * BN);
             bfrag[i][2 * t] = v[0];
             bfrag[i][2 * t + 1] = v[1];
         }
     };
-    auto read_afrag = [&](int buf, int j, uint32_t stage_base) {
+    auto read_afrag = [&](int buf, int j, int stage) {
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-            i32x2 v = rd(stage_base, (aoff_base ^ (j << 4)) + t * 8 * BM);
+            i32x2 v = rd(stage * STAGE_A, (aoff_base ^ (j << 4)) + t * 8 * BM);
             afrag[buf][2 * t] = v[0];
             afrag[buf][2 * t + 1] = v[1];
         }
     };
-    auto read_scales = [&](uint32_t stage_base) {
+    auto read_scales = [&](int stage) {
 #pragma unroll
         for (int q = 0; q < TM / 4; q++) {
-            f32x4 v = *(RF_LDS f32x4 *)(lds + stage_base + soff + q * 16);
+            f32x4 v = *(RF_LDS f32x4 *)(lds + stage * STAGE_S + soff + q * 16);
 #pragma unroll
             for (int e = 0; e < 4; e++) sraw[4 * q + e] = v[e];
         }
@@ -310,15 +317,16 @@ __device__ __forceinline__ void tile_mainloop(
 #pragma unroll
         for (int i = 1; i < TN; i++) read_bfrag(i, 0);
 #pragma unroll
-        for (int d = 0; d < TN && d < NDMA; d++) issue_dma(d, STAGE, dma_src(d, clamp_kb(kb_begin + 1)));
+        for (int d = 0; d < TN && d < NDMA; d++) issue_dma(d, 1, dma_src(d, clamp_kb(kb_begin + 1)));
     }
     // running DMA sources: instructions d >= TN are issued for block kb+1 in the first slots of iteration kb,
     // instructions d < TN for block kb+2 in its last slots (blocks past the end are clamped to the last one)
     const uint8_t *dsrc[NDMA];
 #pragma unroll
     for (int d = 0; d < NDMA; d++) dsrc[d] = dma_src(d, clamp_kb(kb_begin + (d < TN ? 2 : 1)));
-    for (int kb = kb_begin, it = 0; kb < kb_end; ++kb, ++it) {
-        const uint32_t cur = (it & 1) * STAGE, nxt = ((it + 1) & 1) * STAGE;
+    // one K block; CUR is the stage it reads (a compile-time 0 or 1: the loop below is unrolled by two)
+    auto k_block = [&](auto cur_c, int kb) {
+        constexpr int cur = decltype(cur_c)::value, nxt = 1 - cur;
         const int kn1 = clamp_kb(kb + 1);
         const bool adv1 = kb + 2 <= kb_last, adv2 = kb + 3 <= kb_last;   // does the next iteration move on a block?
         const float s_last = s[TM - 1];                    // scale of the previous block's last m-tile (lagged folds)
@@ -379,7 +387,13 @@ __device__ __forceinline__ void tile_mainloop(
             __builtin_amdgcn_sched_barrier(0);
         }
         sb_cur = sb_next;
+    };
+    int kb = kb_begin;
+    for (; kb + 1 < kb_end; kb += 2) {
+        k_block(IntTag<0>{}, kb);
+        k_block(IntTag<1>{}, kb + 1);
     }
+    if (kb < kb_end) k_block(IntTag<0>{}, kb);
     // folds still owed by the last K block
 #pragma unroll
     for (int t = 0; t < LAG; t++) {
