@@ -34,6 +34,8 @@ CONFIGS = {
     "C5": (1024, 576, 7168, 12346),
 }
 RTOL, ATOL, ATOL_REFERENCE = 2e-2, 1e-2, 1e-3
+TRAFFIC_C2_BYTES = 394.2e6
+TRAFFIC_C2_NOTE = "fetch 337.6 MB + write 56.6 MB per launch, profiles/gemm_fp8_blockscale_persistent_C2_hbm_traffic.txt"
 
 
 def algorithmic_bytes(m, n, k):
@@ -156,11 +158,12 @@ def main():
         roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                     "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}
     # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, scaled by a copy
-    # kernel (profiles/gemm_fp8_blockscale_tile_C2_hbm_traffic.txt); only known for the headline plan
-    if args.config == "C2" and (cfg.variant, cfg.split_k, cfg.stream_k) == (0, 1, 0):
-        roofline["traffic"] = 385.4e6
-        roofline["traffic_note"] = "fetch 328.8 MB + write 56.6 MB per launch, profiles/gemm_fp8_blockscale_tile_C2_hbm_traffic.txt"
-    roofline["kernel"] = "gemm_fp8_blockscale_tile (variant %d, split_k %d)" % (cfg.variant, cfg.split_k)
+    # kernel (profiles/gemm_fp8_blockscale_persistent_C2_hbm_traffic.txt); only known for the headline plan
+    if args.config == "C2" and (cfg.variant, cfg.split_k, cfg.stream_k) == (0, 1, 2):
+        roofline["traffic"] = TRAFFIC_C2_BYTES
+        roofline["traffic_note"] = TRAFFIC_C2_NOTE
+    schedule = {0: "gemm_fp8_blockscale_tile", 1: "gemm_fp8_blockscale_streamk", 2: "gemm_fp8_blockscale_persistent"}
+    roofline["kernel"] = "%s (variant %d, split_k %d)" % (schedule.get(cfg.stream_k, "?"), cfg.variant, cfg.split_k)
     roofline["avg_launch_us"] = round(us, 2)
     roofline["algorithmic_flop_per_launch"] = flop
     roofline["algorithmic_bytes_per_launch"] = algorithmic_bytes(m, n, k)

@@ -38,14 +38,21 @@ enum {
     RF_ERR_BAD_CONFIG = 4      /* explicit config not available for this shape */
 };
 
+enum { RF_SCHEDULE_TILES = 0, RF_SCHEDULE_STREAM_K = 1, RF_SCHEDULE_PERSISTENT = 2 };
+
 /* One launch plan: which kernel variant and how K is split.
  * Replaces a DISPATCH_GEMM(...) line of the reference (src/gemm/gemm_launcher.cpp:158-162,229-259). */
 typedef struct rf_gemm_config {
     int variant;      /* index into the variant table, see rf_gemm_variant_info(); -1 = bounds-checked kernel */
     int split_k;      /* >= 1; K blocks are divided over this many partial sums */
     int group_m;      /* tile-order grouping along M for L2 reuse (>=1) */
-    int stream_k;     /* 1: persistent grid, one workgroup per CU, equal shares of the tile x K-block work line;
-                         needs split_k == 1 and at least as many tiles as CUs. 0: one workgroup per tile */
+    int stream_k;     /* schedule, one of RF_SCHEDULE_*:
+                         0 TILES      one workgroup per tile (and per K split);
+                         1 STREAM_K   persistent grid, one workgroup per CU, equal shares of the tile x K-block work
+                                      line; needs split_k == 1 and at least as many tiles as CUs;
+                         2 PERSISTENT persistent grid, whole tiles, one load/compute pipeline running across the
+                                      tiles of a workgroup; needs split_k == 1, M and N multiples of the tile,
+                                      K/128 even */
 } rf_gemm_config;
 
 /* Drop-in for the reference's launcher entry (src/gemm/gemm_launcher.cpp:182-184):
@@ -73,8 +80,10 @@ int rf_gemm_select_config(int m, int n, int k, rf_gemm_config *out);
 /* Variant table introspection (for the tuner and tests). Returns RF_ERR_BAD_CONFIG past the end. */
 int rf_gemm_num_variants(void);
 int rf_gemm_variant_info(int variant, int *block_m, int *block_n, int *waves_m, int *waves_n, int *lds_bytes);
-/* 1 if the variant can run with rf_gemm_config.stream_k = 1, 0 if not (or if the index is out of range). */
+/* 1 if the variant can run with rf_gemm_config.stream_k = RF_SCHEDULE_STREAM_K / RF_SCHEDULE_PERSISTENT, 0 if not
+ * (or if the index is out of range). */
 int rf_gemm_variant_has_stream_k(int variant);
+int rf_gemm_variant_has_persistent(int variant);
 
 /* Device workspace (split-K partial sums) needed for a shape under the automatic plan, in bytes. */
 size_t rf_gemm_workspace_bytes(int m, int n, int k);

@@ -408,19 +408,29 @@ __device__ __forceinline__ void tile_mainloop(
 
 // Stores a wave's accumulators as bf16 into C, masked at the M and N edges. In the MFMA layout a lane owns 4
 // consecutive n of one row, so a direct store instruction would touch 16 rows with 32-byte pieces. Instead each wave
-// stages its tile through its own LDS region (row = WN bf16 + 16 bytes of padding) and writes it back out with
-// 16 bytes per lane, 8 lanes per row: every store instruction covers whole 128-byte lines.
-// All waves must call it together: it starts with a barrier, because LDS-DMA loads of other waves may still be
-// landing in the stage buffers that are reused here.
-template <int BM, int BN, int WAVES_M, int WAVES_N>
-__device__ __forceinline__ void store_tile_bf16(const f32x4 (&acc)[BM / WAVES_M / 16][BN / WAVES_N / 16],
-                                                uint16_t *__restrict__ C, int M, int N, int m0, int n0, uint8_t *lds) {
+// stages its tile, TM/PASSES m-tiles at a time, through its own LDS region (row = WN bf16 + 16 bytes of padding) and
+// writes it back out with 16 bytes per lane, 8 lanes per row: every store instruction covers whole 128-byte lines.
+// `staging` is the start of NW regions of StoreGeom::REGION bytes. BARRIER: the regions overlay the stage buffers,
+// so all waves must call together and a barrier comes first (LDS-DMA loads of other waves may still be landing
+// there). Without it the regions are private memory of the waves and nothing is synchronised.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int PASSES>
+struct StoreGeom {
     using G = TileGeom<BM, BN, WAVES_M, WAVES_N>;
-    constexpr int ROW = G::WN * 2 + 16;                  // bytes per staged row
-    constexpr int HALF_TM = G::TM / 2, ROWS = HALF_TM * 16;
+    static constexpr int ROW = G::WN * 2 + 16;           // bytes per staged row
+    static constexpr int ROWS = G::TM / PASSES * 16;     // rows staged per pass
+    static constexpr int REGION = ROWS * ROW;            // bytes per wave
+    static_assert(G::TM % PASSES == 0, "whole m-tiles per pass");
+};
+template <int BM, int BN, int WAVES_M, int WAVES_N, int PASSES = 2, bool BARRIER = true>
+__device__ __forceinline__ void store_tile_bf16(const f32x4 (&acc)[BM / WAVES_M / 16][BN / WAVES_N / 16],
+                                                uint16_t *__restrict__ C, int M, int N, int m0, int n0,
+                                                uint8_t *staging) {
+    using G = TileGeom<BM, BN, WAVES_M, WAVES_N>;
+    using S = StoreGeom<BM, BN, WAVES_M, WAVES_N, PASSES>;
+    constexpr int ROW = S::ROW, ROWS = S::ROWS, TMP = G::TM / PASSES;
     constexpr int LPR = G::WN * 2 / 16;                  // lanes per row on the way out (16 bytes each)
     constexpr int RPI = 64 / LPR;                        // rows per store instruction
-    static_assert(G::NW * ROWS * ROW <= 2 * G::STAGE, "staging fits in the stage buffers");
+    static_assert(!BARRIER || G::NW * S::REGION <= 2 * G::STAGE, "staging fits in the stage buffers");
     static_assert(ROWS % RPI == 0, "whole store instructions");
     // the opaque zero keeps this address arithmetic below the main loop: hoisted above it, it would cost the
     // loop dozens of registers
@@ -428,13 +438,13 @@ __device__ __forceinline__ void store_tile_bf16(const f32x4 (&acc)[BM / WAVES_M 
     asm volatile("v_mov_b32 %0, 0" : "=v"(vz));
     const int lane = (threadIdx.x & 63) + vz, wave = threadIdx.x >> 6, L = lane & 15, g = lane >> 4;
     const int wm = wave % WAVES_M, wn = wave / WAVES_M;
-    uint8_t *region = lds + wave * (ROWS * ROW);
-    __syncthreads();
+    uint8_t *region = staging + wave * S::REGION;
+    if constexpr (BARRIER) __syncthreads();
 #pragma unroll
-    for (int h = 0; h < 2; h++) {
+    for (int h = 0; h < PASSES; h++) {
 #pragma unroll
-        for (int jj = 0; jj < HALF_TM; jj++) {
-            const int j = h * HALF_TM + jj;
+        for (int jj = 0; jj < TMP; jj++) {
+            const int j = h * TMP + jj;
 #pragma unroll
             for (int i = 0; i < G::TN; i++) {            // lane holds C[16j + L][16i + 4g .. +3]
                 uint2 v;
@@ -446,7 +456,7 @@ __device__ __forceinline__ void store_tile_bf16(const f32x4 (&acc)[BM / WAVES_M 
         // same wave writes and reads its region: program order is enough, the compiler inserts the LDS wait
 #pragma unroll
         for (int r0 = 0; r0 < ROWS; r0 += RPI) {
-            const int r = r0 + lane / LPR, cb = (lane % LPR) * 16;          // row in the half, byte column
+            const int r = r0 + lane / LPR, cb = (lane % LPR) * 16;          // row in the pass, byte column
             const uint4 v = *(const uint4 *)(region + r * ROW + cb);
             const int m = m0 + wm * G::WM + h * ROWS + r;
             const int n = n0 + wn * G::WN + cb / 2;

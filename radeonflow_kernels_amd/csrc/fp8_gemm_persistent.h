@@ -1,0 +1,315 @@
+// Persistent form of gemm_fp8_blockscale_tile: one workgroup per compute unit walks its tiles (id, id + grid,
+// id + 2*grid, ...) and runs ONE software pipeline over the concatenated K blocks of all of them.
+//
+// What it buys: in the one-workgroup-per-tile kernel every tile pays for a cold start (first stage loaded with
+// nothing to overlap, ~2 us), for two redundant prefetches at its end and for a workgroup launch. Here the loads of
+// the next tile's first two K blocks are simply the next loads of the pipeline: they are in flight while the last
+// K blocks of the current tile compute, its first fragments are fetched in the last slots of the current tile, and
+// the bf16 store of the finished tile runs from a private LDS region while the next stage is already resident.
+// Tiles with few K blocks (K = 256: two per tile) gain the most.
+//
+// Restrictions (checked by the host): M % BM == 0 and N % BN == 0 (per-lane load offsets are tile-independent, the
+// tile origin lives in the scalar base pointers), K/128 even (a tile starts on LDS stage 0). Numerics and the
+// per-tile instruction schedule are those of tile_mainloop.
+#pragma once
+#include "fp8_gemm_kernels.h"
+
+namespace rf {
+
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+struct PersistentGeom {
+    using G = TileGeom<BM, BN, WAVES_M, WAVES_N>;
+    static constexpr int STORE_PASSES = G::TM;           // one m-tile (16 rows) per pass: 2.25 KiB per wave
+    using S = StoreGeom<BM, BN, WAVES_M, WAVES_N, STORE_PASSES>;
+    static constexpr int STAGING_OFF = 2 * G::STAGE + 16;
+    static constexpr int LDS_BYTES = STAGING_OFF + G::NW * S::REGION;
+    static_assert(LDS_BYTES <= 160 * 1024, "stages + private store regions fit the CU's LDS");
+};
+
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_persistent(
+    const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
+    const float *__restrict__ SB, uint16_t *__restrict__ C, int M, int N, int K, int tiles_m, int tiles_n,
+    int group_m) {
+    using G = TileGeom<BM, BN, WAVES_M, WAVES_N>;
+    using P = PersistentGeom<BM, BN, WAVES_M, WAVES_N>;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    constexpr int NW = G::NW, WM = G::WM, WN = G::WN, TM = G::TM, TN = G::TN;
+    constexpr int STAGE_A = BK * BM, STAGE_B = BK * BN, STAGE_S = BM * 4;
+    constexpr int OFF_B = 2 * STAGE_A, OFF_S = 2 * STAGE_A + 2 * STAGE_B;
+    static_assert(STAGE_A + 3 * 8 * BM + 16 * (BM / 16) < 65536 && STAGE_B + 3 * 8 * BN + 16 * (BN / 16) < 65536,
+                  "stage offsets must fit the immediate offset of an LDS read");
+    constexpr int INST_A = STAGE_A / 1024 / NW, INST_B = STAGE_B / 1024 / NW;
+    constexpr int NSC = BM / 64;
+    static_assert(STAGE_A % (1024 * NW) == 0 && STAGE_B % (1024 * NW) == 0, "loads must divide evenly over waves");
+    static_assert(NSC <= NW && WN <= 128 && 128 % WN == 0 && TM % 4 == 0, "same tile constraints as tile_mainloop");
+    constexpr int CPR_A = BM / 16, CPR_B = BN / 16, RPI_A = 1024 / BM, RPI_B = 1024 / BN;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int L = lane & 15, g = lane >> 4;
+    const int wm = wave % WAVES_M, wn = wave / WAVES_M;
+    const int QK = K / BK, QN = (N + 127) / 128;
+    const int T = tiles_m * tiles_n;
+    const int my_tiles =                                                                // >= 1: grid <= T
+        __builtin_amdgcn_readfirstlane((T - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x);
+
+    // origin of this workgroup's r-th tile; past the end it repeats the last one (prefetches that nobody uses)
+    auto tile_origin = [&](int r, int &m0, int &n0) {
+        if (r > my_tiles - 1) r = my_tiles - 1;
+        int tm, tn;
+        tile_of_block(blockIdx.x + r * gridDim.x, T, tiles_m, tiles_n, group_m, true, tm, tn);
+        // the divisions above run on the vector unit; the origins feed scalar base pointers
+        m0 = __builtin_amdgcn_readfirstlane(tm * BM);
+        n0 = __builtin_amdgcn_readfirstlane(tn * BN);
+    };
+
+    // ---- global -> LDS: per-lane offsets inside a K block, relative to the tile origin (see tile_mainloop) ----
+    constexpr int PER_A = (8 / RPI_A) > 0 ? (8 / RPI_A) : 1, PER_B = (8 / RPI_B) > 0 ? (8 / RPI_B) : 1;
+    constexpr int GRP_A = (INST_A * RPI_A + 31) / 32, GRP_B = (INST_B * RPI_B + 31) / 32;
+    constexpr int NCLS_A = (PER_A < INST_A ? PER_A : INST_A) * GRP_A, NCLS_B = (PER_B < INST_B ? PER_B : INST_B) * GRP_B;
+    static_assert((INST_A * RPI_A) % 32 == 0 || INST_A * RPI_A < 32, "a wave's rows cover whole 32-row groups");
+    static_assert((INST_B * RPI_B) % 32 == 0 || INST_B * RPI_B < 32, "a wave's rows cover whole 32-row groups");
+    auto cls_a = [](int i) { return i % PER_A + PER_A * (i * RPI_A / 32); };
+    auto rep_a = [](int c) { return c % PER_A + (c / PER_A) * (32 / RPI_A); };
+    auto cls_b = [](int i) { return i % PER_B + PER_B * (i * RPI_B / 32); };
+    auto rep_b = [](int c) { return c % PER_B + (c / PER_B) * (32 / RPI_B); };
+    uint32_t goff_a[NCLS_A], goff_b[NCLS_B], goff_s;
+#pragma unroll
+    for (int c_ = 0; c_ < NCLS_A; c_++) {
+        const int kl = (wave * INST_A + rep_a(c_)) * RPI_A + lane / CPR_A;
+        const int c = (lane % CPR_A) ^ swizzle_of_row<BM>(kl);
+        goff_a[c_] = (uint32_t)(lane / CPR_A) * (uint32_t)M + (uint32_t)(c * 16);
+    }
+#pragma unroll
+    for (int c_ = 0; c_ < NCLS_B; c_++) {
+        const int kl = (wave * INST_B + rep_b(c_)) * RPI_B + lane / CPR_B;
+        const int c = (lane % CPR_B) ^ swizzle_of_row<BN>(kl);
+        goff_b[c_] = (uint32_t)(lane / CPR_B) * (uint32_t)N + (uint32_t)(c * 16);
+    }
+    {
+        const int sl = (wave < NSC ? wave : 0) * 64 + lane, r = sl % WM;
+        goff_s = (uint32_t)((sl / WM) * WM + 16 * (r % TM) + r / TM) * 4u;
+    }
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(RF_LDS uint8_t *)lds;
+    constexpr int NDMA = INST_A + INST_B + 1;
+    const uint32_t lds_dst_a = lds_base + wave * (INST_A * 1024), lds_dst_b = lds_base + OFF_B + wave * (INST_B * 1024),
+                   lds_dst_s = lds_base + OFF_S + wave * 256;
+    auto dma_src = [&](int d, int m0, int n0, int kb) -> const uint8_t * {
+        if (d < INST_A) return A + ((size_t)kb * BK + (size_t)(wave * INST_A + d) * RPI_A) * M + m0;
+        if (d < INST_A + INST_B) return B + ((size_t)kb * BK + (size_t)(wave * INST_B + (d - INST_A)) * RPI_B) * N + n0;
+        return (const uint8_t *)(SA + (size_t)kb * M + m0);
+    };
+    auto dma_step = [&](int d) -> size_t {
+        return d < INST_A ? (size_t)BK * M : d < INST_A + INST_B ? (size_t)BK * N : (size_t)M * 4;
+    };
+    auto issue_dma = [&](int d, int stage, const uint8_t *src) {
+        if (d < INST_A) {
+            asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                         :: "v"(goff_a[cls_a(d < INST_A ? d : 0)]), "s"(src), "s"(lds_dst_a), "n"(d * 1024 + stage * STAGE_A)
+                         : "memory", "scc");
+        } else if (d < INST_A + INST_B) {
+            const int e = d - INST_A < INST_B ? d - INST_A : 0;
+            asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                         :: "v"(goff_b[cls_b(e >= 0 ? e : 0)]), "s"(src), "s"(lds_dst_b), "n"(e * 1024 + stage * STAGE_B)
+                         : "memory", "scc");
+        } else if (wave < NSC) {
+            asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+                         :: "v"(goff_s), "s"(src), "s"(lds_dst_s), "n"(stage * STAGE_S) : "memory", "scc");
+        }
+    };
+
+    // ---- LDS -> MFMA operands (see tile_mainloop) ----
+    const int krow = 32 * g + (L >> 1);
+    static_assert((TM & (TM - 1)) == 0 && (TN & (TN - 1)) == 0, "tile counts are powers of two");
+    const uint32_t aoff_base = krow * BM + (((wm * TM) ^ swizzle_of_row<BM>(krow)) << 4) + 8 * (L & 1);
+    const uint32_t boff_base = OFF_B + krow * BN + (((wn * TN) ^ swizzle_of_row<BN>(krow)) << 4) + 8 * (L & 1);
+    const uint32_t soff = OFF_S + (wm * WM + L * TM) * 4;
+
+    int vzero;
+    asm volatile("v_mov_b32 %0, 0" : "=v"(vzero));
+
+    constexpr int PR = 4, LAG = 3, NMFMA = TM * TN, BAR_SLOT = (TM - 1) * TN;
+    static_assert(LAG < TN && LAG < PR && TM % 2 == 0 && NDMA - TN <= BAR_SLOT, "same schedule as tile_mainloop");
+
+    f32x4 acc[TM][TN];
+    i32x8 bfrag[TN], afrag[2];
+    f32x4 pring[PR];
+    float s[TM], sraw[TM], sb_cur = 0.f, sb_next = 0.f;
+#pragma unroll
+    for (int j = 0; j < TM; j++)
+#pragma unroll
+        for (int i = 0; i < TN; i++) acc[j][i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int r = 0; r < PR; r++) pring[r] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < TM; j++) s[j] = 0.f;
+
+    auto rd = [&](uint32_t stage_base, uint32_t off) {
+        return __builtin_amdgcn_ds_read_tr8_b64_v2i32((RF_LDS i32x2 *)(lds + stage_base + off));
+    };
+    auto read_bfrag = [&](int i, int stage) {
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            i32x2 v = rd(stage * STAGE_B, (boff_base ^ (i << 4)) + t * 8 * BN);
+            bfrag[i][2 * t] = v[0];
+            bfrag[i][2 * t + 1] = v[1];
+        }
+    };
+    auto read_afrag = [&](int buf, int j, int stage) {
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            i32x2 v = rd(stage * STAGE_A, (aoff_base ^ (j << 4)) + t * 8 * BM);
+            afrag[buf][2 * t] = v[0];
+            afrag[buf][2 * t + 1] = v[1];
+        }
+    };
+    auto read_scales = [&](int stage) {
+#pragma unroll
+        for (int q = 0; q < TM / 4; q++) {
+            f32x4 v = *(RF_LDS f32x4 *)(lds + stage * STAGE_S + soff + q * 16);
+#pragma unroll
+            for (int e = 0; e < 4; e++) sraw[4 * q + e] = v[e];
+        }
+    };
+
+    // ---- two load cursors run ahead of the compute position ----
+    // cursor 1 = the K block after the current one (DMA instructions d >= TN, issued in the first slots of a step, and
+    // the b_scale load); cursor 2 = two blocks ahead (instructions d < TN, issued after the barrier). Each holds its
+    // tile ordinal, K block and the running source pointers of its instructions; crossing into the next tile
+    // recomputes the pointers from that tile's origin.
+    const uint8_t *dsrc[NDMA];
+    int c1_r = 0, c1_kb = 0, c2_r = 0, c2_kb = 0;     // set below
+    int sb_off1 = 0;                                  // index into SB of cursor 1's block for this wave's columns
+    auto nb_of = [&](int n0) { return (n0 + wn * WN) >> 7; };
+    auto seek = [&](bool first_group, int r, int kb) {   // point a cursor's instructions at (tile r, block kb)
+        int m0, n0;
+        tile_origin(r, m0, n0);
+#pragma unroll
+        for (int d = 0; d < NDMA; d++)
+            if ((d >= TN) == first_group) dsrc[d] = dma_src(d, m0, n0, kb);
+        if (first_group) sb_off1 = kb * QN + nb_of(n0);
+    };
+    auto advance = [&](bool first_group, int &r, int &kb) {   // move a cursor one K block on
+        if (kb + 1 < QK) {
+            kb += 1;
+#pragma unroll
+            for (int d = 0; d < NDMA; d++)
+                if ((d >= TN) == first_group) dsrc[d] += dma_step(d);
+            if (first_group) sb_off1 += QN;
+        } else {
+            r += 1;
+            kb = 0;
+            seek(first_group, r, 0);
+        }
+    };
+
+    int m0_cur, n0_cur;
+    tile_origin(0, m0_cur, n0_cur);
+    {
+        // cold start: stage 0 <- block 0 of the first tile, then its first operands; stage 1 <- start of block 1
+#pragma unroll
+        for (int d = 0; d < NDMA; d++) issue_dma(d, 0, dma_src(d, m0_cur, n0_cur, 0));
+        sb_cur = SB[nb_of(n0_cur) + vzero];
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        asm volatile("" : "+v"(sb_cur));
+        __syncthreads();
+        read_bfrag(0, 0);
+        read_afrag(0, 0, 0);
+        read_scales(0);
+#pragma unroll
+        for (int i = 1; i < TN; i++) read_bfrag(i, 0);
+        // cursor 1 at block 1 (QK >= 2); its instructions d < TN ... belong to cursor 2, which starts at block 1 too
+        // for this one partial batch and then moves on to block 2
+        c2_r = 0; c2_kb = 1;
+        seek(false, 0, 1);
+#pragma unroll
+        for (int d = 0; d < TN && d < NDMA; d++) issue_dma(d, 1, dsrc[d]);
+        advance(false, c2_r, c2_kb);                  // cursor 2 -> block 2 (or the next tile)
+        c1_r = 0; c1_kb = 1;
+        seek(true, 0, 1);
+    }
+
+    // one K block of the current tile; cur = the LDS stage it reads
+    auto k_block = [&](auto cur_c) {
+        constexpr int cur = decltype(cur_c)::value, nxt = 1 - cur;
+        const float s_last = s[TM - 1];
+#pragma unroll
+        for (int j = 0; j < TM; j++) s[j] = sraw[j] * sb_cur;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < NMFMA; t++) {
+            const int j = t / TN, i = t % TN;
+            if (t == BAR_SLOT) {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                asm volatile("" : "+v"(sb_next));
+                __syncthreads();
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (t == 0) sb_next = SB[sb_off1 + vzero];
+            pring[t % PR] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                bfrag[i], afrag[j & 1], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+            asm volatile("" : "+v"(pring[t % PR]));
+            __builtin_amdgcn_sched_barrier(0);
+            if (t + TN < NDMA) issue_dma(t + TN, nxt, dsrc[t + TN]);                       // cursor 1
+            if (t >= BAR_SLOT && t - BAR_SLOT < NDMA && t - BAR_SLOT < TN)
+                issue_dma(t - BAR_SLOT, cur, dsrc[t - BAR_SLOT]);                          // cursor 2
+            if (j + 1 < TM) {
+                if (i == 0) read_afrag((j + 1) & 1, j + 1, cur);
+            } else {
+                read_bfrag(i, nxt);
+                if (i == 0) {
+                    read_afrag(0, 0, nxt);
+                    read_scales(nxt);
+                }
+            }
+            if (t >= LAG) {
+                const int u = t - LAG, ju = u / TN, iu = u % TN;
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[ju][iu][e] = __builtin_fmaf(s[ju], pring[u % PR][e], acc[ju][iu][e]);
+                asm volatile("" : "+v"(acc[ju][iu]));
+            } else {
+                const int u = NMFMA + t - LAG, ju = u / TN, iu = u % TN;
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[ju][iu][e] = __builtin_fmaf(s_last, pring[u % PR][e], acc[ju][iu][e]);
+                asm volatile("" : "+v"(acc[ju][iu]));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        sb_cur = sb_next;
+        advance(true, c1_r, c1_kb);
+        advance(false, c2_r, c2_kb);
+    };
+
+    for (int r = 0; r < my_tiles; r++) {
+        for (int kb = 0; kb < QK; kb += 2) {
+            k_block(IntTag<0>{});
+            k_block(IntTag<1>{});
+        }
+        // the tile is complete: fold what the last K block still owes, store, start the next tile from zero. The
+        // operands of the next tile's first K block are already in registers, its second block is on its way.
+#pragma unroll
+        for (int t = 0; t < LAG; t++) {
+            const int u = NMFMA + t - LAG, ju = u / TN, iu = u % TN;
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[ju][iu][e] = __builtin_fmaf(s[TM - 1], pring[u % PR][e], acc[ju][iu][e]);
+        }
+        store_tile_bf16<BM, BN, WAVES_M, WAVES_N, P::STORE_PASSES, false>(acc, C, M, N, m0_cur, n0_cur,
+                                                                          lds + P::STAGING_OFF);
+#pragma unroll
+        for (int j = 0; j < TM; j++)
+#pragma unroll
+            for (int i = 0; i < TN; i++) acc[j][i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        // the first LAG folds of the next K block add s[TM-1] * (ring entries of this tile): make that 0 * 0
+#pragma unroll
+        for (int q = 0; q < PR; q++) pring[q] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < TM; j++) s[j] = 0.f;
+        tile_origin(r + 1, m0_cur, n0_cur);
+    }
+    // prefetches past the last tile must land before the LDS is handed on
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+}  // namespace rf

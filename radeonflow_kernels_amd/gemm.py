@@ -38,7 +38,7 @@ class PerfMetrics(ctypes.Structure):
 
 
 EXPORTS = ("run", "rf_fp8_gemm", "rf_fp8_gemm_ex", "rf_gemm_select_config", "rf_gemm_num_variants",
-           "rf_gemm_variant_info", "rf_gemm_variant_has_stream_k", "rf_gemm_workspace_bytes", "rf_gemm_init", "rf_gemm_destroy",
+           "rf_gemm_variant_info", "rf_gemm_variant_has_stream_k", "rf_gemm_variant_has_persistent", "rf_gemm_workspace_bytes", "rf_gemm_init", "rf_gemm_destroy",
            "rf_gemm_last_error", "rf_quantize_a_f32", "rf_quantize_a_bf16", "rf_quantize_b_f32", "rf_quantize_b_bf16")
 
 
@@ -64,6 +64,8 @@ def lib():
         L.rf_gemm_variant_info.restype = i32
         L.rf_gemm_variant_has_stream_k.argtypes = [i32]
         L.rf_gemm_variant_has_stream_k.restype = i32
+        L.rf_gemm_variant_has_persistent.argtypes = [i32]
+        L.rf_gemm_variant_has_persistent.restype = i32
         L.rf_gemm_workspace_bytes.argtypes = [i32, i32, i32]
         L.rf_gemm_workspace_bytes.restype = ctypes.c_size_t
         L.rf_gemm_init.argtypes = [ctypes.c_size_t]
@@ -180,5 +182,6 @@ def variants():
         L.rf_gemm_variant_info(v, *[ctypes.byref(x) for x in vals])
         out.append(dict(variant=v, block_m=vals[0].value, block_n=vals[1].value, waves_m=vals[2].value,
                         waves_n=vals[3].value, lds_bytes=vals[4].value,
-                        stream_k=bool(L.rf_gemm_variant_has_stream_k(v))))
+                        stream_k=bool(L.rf_gemm_variant_has_stream_k(v)),
+                        persistent=bool(L.rf_gemm_variant_has_persistent(v))))
     return out

@@ -77,8 +77,11 @@ def tune_shape(rfk, m, n, k, log=print):
     ncu = torch.cuda.get_device_properties(0).multi_processor_count
     for v in rfk.variants():
         tiles = -(-m // v["block_m"]) * -(-n // v["block_n"])
-        for split, sk in [(sp, 0) for sp in SPLITS] + [(1, 1)]:
-            if split > k // 128 or (sk and tiles < ncu):
+        # schedules: 0 = one workgroup per tile (with K splits), 1 = stream-K, 2 = persistent whole tiles
+        for split, sk in [(sp, 0) for sp in SPLITS] + [(1, 1), (1, 2)]:
+            if split > k // 128 or (sk == 1 and (tiles < ncu or not v["stream_k"])):
+                continue
+            if sk == 2 and (not v["persistent"] or m % v["block_m"] or n % v["block_n"] or (k // 128) % 2):
                 continue
             for gm in GROUPS:
                 cfg = rfk.GemmConfig(v["variant"], split, gm, sk)

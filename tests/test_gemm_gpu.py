@@ -108,6 +108,36 @@ def test_stream_k_bit_exact_and_counters_self_reset(rfk, m, n, k):
     assert tried > 0
 
 
+@pytest.mark.parametrize("m,n,k", [(512, 512, 256), (2048, 2048, 512), (2560, 1920, 256), (6144, 4608, 256),
+                                   (4096, 2048, 1024), (1024, 1536, 7168)])
+def test_persistent_schedule_bit_exact(rfk, m, n, k):
+    """One pipeline running across the tiles of a workgroup (1, 2 or 3 tiles each, uneven counts included): exact
+    data, so every tile must equal the oracle bit for bit whatever was prefetched or left in registers by the
+    previous tile. Twice in a row on the same buffers."""
+    data = exact_problem(m, n, k, seed=5 * m + n + k)
+    exp = oracle_bf16(data)
+    tried = 0
+    for v in rfk.variants():
+        if not v["persistent"] or m % v["block_m"] or n % v["block_n"]:
+            continue
+        for gm in (1, 8):
+            cfg = rfk.GemmConfig(v["variant"], 1, gm, 2)
+            for rep in range(2):
+                out = _run(rfk, data, config=cfg, canary=1024)
+                assert np.array_equal(bf16_bits(out), exp), "plan %r rep %d" % (cfg, rep)
+            tried += 1
+    assert tried > 0
+
+
+def test_persistent_schedule_rejects_ragged_shapes(rfk):
+    data = exact_problem(272, 144, 256, seed=1)
+    with pytest.raises(RuntimeError):
+        _run(rfk, data, config=rfk.GemmConfig(0, 1, 1, 2))
+    data = exact_problem(256, 256, 384, seed=1)           # three K blocks
+    with pytest.raises(RuntimeError):
+        _run(rfk, data, config=rfk.GemmConfig(0, 1, 1, 2))
+
+
 @pytest.mark.parametrize("m,n,k", [(3, 130, 256), (1, 1, 128), (17, 64, 384), (5, 257, 128), (100, 72, 256)])
 def test_bounds_checked_kernel_on_odd_shapes(rfk, m, n, k):
     data = rk.generate_input_reference_style(m, n, k, seed=7 * m + n)
