@@ -101,34 +101,37 @@ __device__ __forceinline__ void tile_of_block(int bid, int nblocks, int tiles_m,
     tile_n = in_grp / rows;
 }
 
-// Geometry of one kernel variant.
-template <int BM_, int BN_, int WAVES_M_, int WAVES_N_>
+// Geometry of one kernel variant. NS = number of LDS stages (K blocks resident or in flight).
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int NS_ = 2>
 struct TileGeom {
-    static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+    static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, NS = NS_;
     static constexpr int NW = WAVES_M * WAVES_N, NT = NW * 64;
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 16, TN = WN / 16;
-    static constexpr int STAGE = BK * BM + BK * BN + BM * 4;      // A rows, B rows, a_scale
-    static constexpr int LDS_BYTES = 2 * STAGE + 16;              // two stages + a 16-byte mailbox
+    static constexpr int STAGE_A = BK * BM, STAGE_B = BK * BN;
+    static constexpr int STAGE_S = BM * 4 + 256;                  // a_scale of the tile rows + 64 b_scale slots
+    static constexpr int STAGE = STAGE_A + STAGE_B + STAGE_S;
+    static constexpr int LDS_BYTES = NS * STAGE + 16;             // the stages + a 16-byte mailbox
+    static_assert(LDS_BYTES <= 160 * 1024, "stages fit the CU's LDS");
 };
 
 // Accumulates into acc the contribution of K blocks [kb_begin, kb_end) to the BM x BN tile at (m0, n0).
 // All waves of the workgroup call it together. On return every LDS-DMA load has landed, but other waves may still
 // be reading LDS: a barrier is needed before LDS is written again.
-template <int BM, int BN, int WAVES_M, int WAVES_N>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NS = 2>
 __device__ __forceinline__ void tile_mainloop(
     const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
     const float *__restrict__ SB, int M, int N, int m0, int n0, int kb_begin, int kb_end, uint8_t *lds,
     f32x4 (&acc)[BM / WAVES_M / 16][BN / WAVES_N / 16]) {
+    using G = TileGeom<BM, BN, WAVES_M, WAVES_N, NS>;
     constexpr int NW = WAVES_M * WAVES_N;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     constexpr int TM = WM / 16, TN = WN / 16;
-    // one LDS stage: A[128][BM] bytes, B[128][BN] bytes and BM fp32 a_scale values. The two stages are interleaved
-    // by operand (A0 A1 B0 B1 S0 S1), so that a transpose read of either stage is "per-lane base register + a
-    // 16-bit immediate": no address arithmetic in the loop.
-    constexpr int STAGE_A = BK * BM, STAGE_B = BK * BN, STAGE_S = BM * 4, STAGE = STAGE_A + STAGE_B + STAGE_S;
-    constexpr int OFF_B = 2 * STAGE_A, OFF_S = 2 * STAGE_A + 2 * STAGE_B;
-    static_assert(STAGE_A + 3 * 8 * BM + 16 * (BM / 16) < 65536 && STAGE_B + 3 * 8 * BN + 16 * (BN / 16) < 65536,
-                  "stage offsets must fit the immediate offset of an LDS read");
+    // one LDS stage: A[128][BM] bytes, B[128][BN] bytes, BM fp32 a_scale values and the b_scale values of the
+    // tile's columns. The stages are interleaved by operand (A0 A1 .. B0 B1 .. S0 S1 ..), so that a transpose read
+    // of any stage is "per-lane base register + immediate": no address arithmetic in the loop.
+    constexpr int STAGE_A = G::STAGE_A, STAGE_B = G::STAGE_B, STAGE_S = G::STAGE_S;
+    constexpr int OFF_B = NS * STAGE_A, OFF_S = NS * (STAGE_A + STAGE_B), OFF_SB = BM * 4;   // OFF_SB inside an S region
+    static_assert(NS >= 2 && NS <= 4, "two to four stages");
     constexpr int INST_A = STAGE_A / 1024 / NW, INST_B = STAGE_B / 1024 / NW;   // 1 KiB per wave instruction
     constexpr int NSC = BM / 64;                                                // scale loads: 64 floats each
     static_assert(STAGE_A % (1024 * NW) == 0 && STAGE_B % (1024 * NW) == 0, "loads must divide evenly over waves");
@@ -159,7 +162,7 @@ __device__ __forceinline__ void tile_mainloop(
     auto rep_a = [](int c) { return c % PER_A + (c / PER_A) * (32 / RPI_A); }; // first instruction of class c
     auto cls_b = [](int i) { return i % PER_B + PER_B * (i * RPI_B / 32); };
     auto rep_b = [](int c) { return c % PER_B + (c / PER_B) * (32 / RPI_B); };
-    uint32_t goff_a[NCLS_A], goff_b[NCLS_B], goff_s;
+    uint32_t goff_a[NCLS_A], goff_b[NCLS_B], goff_s, goff_sb;
 #pragma unroll
     for (int c_ = 0; c_ < NCLS_A; c_++) {
         int q = wave * INST_A + rep_a(c_);
@@ -186,43 +189,61 @@ __device__ __forceinline__ void tile_mainloop(
         int m = m0 + (sl / WM) * WM + 16 * (r % TM) + r / TM;
         if (m > M - 1) m = M - 1;
         goff_s = (uint32_t)m * 4u;
+        // b_scale slot l of the stage holds the scale of the l-th 128-column block the tile touches (clamped)
+        int nbq = (n0 >> 7) + lane;
+        if (nbq > QN - 1) nbq = QN - 1;
+        goff_sb = (uint32_t)nbq * 4u;
     }
     // The LDS-DMA loads are issued through inline asm on purpose: the compiler cannot tell which stage a
     // transpose read touches, so for builtin LDS-DMA loads it waits for vmcnt(0) before the first LDS read
     // that follows them, which serialises the prefetch with the compute it is meant to overlap. Here the
-    // kernel owns the wait: one s_waitcnt vmcnt(0) before the barrier at the top of the next iteration.
+    // kernel owns the wait: one s_waitcnt vmcnt before the barrier of each iteration. For the same reason the loop
+    // contains no other vector memory load at all (the b_scale values come through LDS like the a_scale ones): the
+    // compiler then never emits a vmcnt wait of its own inside it.
     // Addressing: 64-bit SGPR base (advances by 128 rows per K block) + per-lane 32-bit offset; M0 holds
     // the LDS destination of the instruction (lane l lands at M0 + 16*l, or M0 + 4*l for the dword form).
     const uint32_t lds_base = (uint32_t)(uintptr_t)(RF_LDS uint8_t *)lds;
-    constexpr int NDMA = INST_A + INST_B + 1;
-    // DMA instruction d of this wave: A rows (d < INST_A), then B rows, then the scales. Its global source for K
-    // block kb is dma_src(d, kb); its LDS destination inside a stage is fixed. In the loop each instruction keeps a
-    // running source pointer (one 64-bit scalar add per K block) instead of recomputing products.
+    constexpr int D_SA = INST_A + INST_B, D_SB = D_SA + 1, NDMA = D_SB + 1;
+    // DMA instruction d of this wave: A rows (d < INST_A), then B rows, then the a_scales (first NSC waves), then the
+    // b_scales (wave 0). Its global source for K block kb is dma_src(d, kb); its LDS destination inside a stage is
+    // fixed. In the loop each instruction keeps a running source pointer (one 64-bit scalar add per K block).
     const uint32_t lds_dst_a = lds_base + wave * (INST_A * 1024), lds_dst_b = lds_base + OFF_B + wave * (INST_B * 1024),
-                   lds_dst_s = lds_base + OFF_S + wave * 256;
+                   lds_dst_s = lds_base + OFF_S + wave * 256, lds_dst_sb = lds_base + OFF_S + OFF_SB;
     auto dma_src = [&](int d, int kb) -> const uint8_t * {
         if (d < INST_A) return A + ((size_t)kb * BK + (size_t)(wave * INST_A + d) * RPI_A) * M;
-        if (d < INST_A + INST_B) return B + ((size_t)kb * BK + (size_t)(wave * INST_B + (d - INST_A)) * RPI_B) * N;
-        return (const uint8_t *)(SA + (size_t)kb * M);
+        if (d < D_SA) return B + ((size_t)kb * BK + (size_t)(wave * INST_B + (d - INST_A)) * RPI_B) * N;
+        if (d == D_SA) return (const uint8_t *)(SA + (size_t)kb * M);
+        return (const uint8_t *)(SB + (size_t)kb * QN);
     };
     auto dma_step = [&](int d) -> size_t {       // bytes from one K block to the next
-        return d < INST_A ? (size_t)BK * M : d < INST_A + INST_B ? (size_t)BK * N : (size_t)M * 4;
+        return d < INST_A ? (size_t)BK * M : d < D_SA ? (size_t)BK * N : d == D_SA ? (size_t)M * 4 : (size_t)QN * 4;
     };
     auto issue_dma = [&](int d, int stage, const uint8_t *src) {
         if (d < INST_A) {
             asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                          :: "v"(goff_a[cls_a(d < INST_A ? d : 0)]), "s"(src), "s"(lds_dst_a), "n"(d * 1024 + stage * STAGE_A)
                          : "memory", "scc");
-        } else if (d < INST_A + INST_B) {
+        } else if (d < D_SA) {
             const int e = d - INST_A < INST_B ? d - INST_A : 0;
             asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                          :: "v"(goff_b[cls_b(e >= 0 ? e : 0)]), "s"(src), "s"(lds_dst_b), "n"(e * 1024 + stage * STAGE_B)
                          : "memory", "scc");
-        } else if (wave < NSC) {
+        } else if (d == D_SA) {
+            if (wave < NSC)
+                asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+                             :: "v"(goff_s), "s"(src), "s"(lds_dst_s), "n"(stage * STAGE_S) : "memory", "scc");
+        } else if (wave == 0) {
             asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
-                         :: "v"(goff_s), "s"(src), "s"(lds_dst_s), "n"(stage * STAGE_S) : "memory", "scc");
+                         :: "v"(goff_sb), "s"(src), "s"(lds_dst_sb), "n"(stage * STAGE_S) : "memory", "scc");
         }
     };
+    // Wait until the loads of every K block except the newest NS-2 have landed. vmcnt counts this wave's loads in
+    // issue order; the optional scale loads are left out of the allowance, which errs on the side of waiting.
+    auto wait_for_stage = [&]() {
+        if constexpr (NS == 2) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(%0)" :: "n"((NS - 2) * (INST_A + INST_B)) : "memory");
+    };
+    static_assert((NS - 2) * (INST_A + INST_B) < 64, "vmcnt is a 6-bit counter");
 
     // ---- LDS -> MFMA operands: per-lane byte offsets of the transpose reads (stage 0, t = 0) ----
     // lane (L,g) of read t points at row k = 32g + 8t + L/2, half (L&1) of 16-byte chunk c.
@@ -234,19 +255,14 @@ __device__ __forceinline__ void tile_mainloop(
     // (OFF_B has no low bits set, so it passes through the XOR with the tile index unchanged)
     const uint32_t boff_base = OFF_B + krow * BN + (((wn * TN) ^ swizzle_of_row<BN>(krow)) << 4) + 8 * (L & 1);
     const uint32_t soff = OFF_S + (wm * WM + L * TM) * 4;               // this lane's TM scales
-
-    int nb = (n0 + wn * WN) >> 7;
-    if (nb > QN - 1) nb = QN - 1;
+    // this wave's b_scale: its columns lie in one 128-column block, the (nb - first block of the tile)-th slot
+    const uint32_t sboff = OFF_S + OFF_SB + ((((n0 + wn * WN) >> 7) - (n0 >> 7)) << 2);
 
 #pragma unroll
     for (int j = 0; j < TM; j++)
 #pragma unroll
         for (int i = 0; i < TN; i++) acc[j][i] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-    // b_scale is wave-uniform, but it is fetched with a vector load on purpose: a scalar load returns out of
-    // order with LDS reads on the same counter and would force every LDS wait in the loop down to zero.
-    int vzero;
-    asm volatile("v_mov_b32 %0, 0" : "=v"(vzero));
     // ---- main loop: one K block per iteration, software-pipelined by hand across iterations ----
     // MFMA slot t = (m-tile j, n-tile i), row-major. In steady state the matrix pipe never waits for a K-block
     // boundary:
@@ -256,10 +272,10 @@ __device__ __forceinline__ void tile_mainloop(
     //   * the barrier that publishes the next stage sits before the LAST m-tile's slots (slot BAR_SLOT). In those
     //     slots each B-matrix fragment is dead as soon as its MFMA has issued and is refilled from the next
     //     stage, together with the first A fragment and the scales of the next K block;
-    //   * after that barrier the stage just consumed is free: the LDS-DMA loads of K block kb+2 start there, one
+    //   * after that barrier the stage just consumed is free: the LDS-DMA loads of K block kb+NS start there, one
     //     per slot, and run on into the first slots of the next iteration.
     // An empty volatile asm after each MFMA / fold anchors it in its slot, sched_barrier(0) keeps the slots apart;
-    // the compiler still places the waitcnts and hazard nops.
+    // the compiler still places the LDS waits and hazard nops.
     constexpr int PR = 4, LAG = 3, NMFMA = TM * TN, BAR_SLOT = (TM - 1) * TN;
     static_assert(LAG < TN && LAG < PR, "lagged folds of a K block stay inside its last m-tile row");
     static_assert(TM % 2 == 0, "the last m-tile uses afrag[1], so afrag[0] is free for the next block");
@@ -269,7 +285,7 @@ __device__ __forceinline__ void tile_mainloop(
 
     i32x8 bfrag[TN], afrag[2];
     f32x4 pring[PR];
-    float s[TM], sraw[TM], sb_cur = 0.f, sb_next = 0.f;
+    float s[TM], sraw[TM], sb_raw = 0.f;
 #pragma unroll
     for (int r = 0; r < PR; r++) pring[r] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -301,15 +317,16 @@ __device__ __forceinline__ void tile_mainloop(
 #pragma unroll
             for (int e = 0; e < 4; e++) sraw[4 * q + e] = v[e];
         }
+        sb_raw = *(RF_LDS float *)(lds + stage * STAGE_S + sboff);
     };
 
     if (kb_begin < kb_end) {
-        // prologue: stage 0 <- first K block, then its first operands; stage 1 <- second K block
+        // prologue: stages 0..NS-2 <- the first K blocks, then the first operands; stage NS-1 <- start of the next
 #pragma unroll
-        for (int d = 0; d < NDMA; d++) issue_dma(d, 0, dma_src(d, kb_begin));
-        sb_cur = SB[(size_t)kb_begin * QN + nb + vzero];
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        asm volatile("" : "+v"(sb_cur));
+        for (int st = 0; st < NS - 1; st++)
+#pragma unroll
+            for (int d = 0; d < NDMA; d++) issue_dma(d, st, dma_src(d, clamp_kb(kb_begin + st)));
+        wait_for_stage();
         __syncthreads();
         read_bfrag(0, 0);
         read_afrag(0, 0, 0);
@@ -317,21 +334,20 @@ __device__ __forceinline__ void tile_mainloop(
 #pragma unroll
         for (int i = 1; i < TN; i++) read_bfrag(i, 0);
 #pragma unroll
-        for (int d = 0; d < TN && d < NDMA; d++) issue_dma(d, 1, dma_src(d, clamp_kb(kb_begin + 1)));
+        for (int d = 0; d < TN && d < NDMA; d++) issue_dma(d, NS - 1, dma_src(d, clamp_kb(kb_begin + NS - 1)));
     }
-    // running DMA sources: instructions d >= TN are issued for block kb+1 in the first slots of iteration kb,
-    // instructions d < TN for block kb+2 in its last slots (blocks past the end are clamped to the last one)
+    // running DMA sources: instructions d >= TN are issued for block kb+NS-1 in the first slots of iteration kb,
+    // instructions d < TN for block kb+NS in its last slots (blocks past the end are clamped to the last one)
     const uint8_t *dsrc[NDMA];
 #pragma unroll
-    for (int d = 0; d < NDMA; d++) dsrc[d] = dma_src(d, clamp_kb(kb_begin + (d < TN ? 2 : 1)));
-    // one K block; CUR is the stage it reads (a compile-time 0 or 1: the loop below is unrolled by two)
+    for (int d = 0; d < NDMA; d++) dsrc[d] = dma_src(d, clamp_kb(kb_begin + (d < TN ? NS : NS - 1)));
+    // one K block; cur is the stage it reads (compile-time: the loop below is unrolled NS times)
     auto k_block = [&](auto cur_c, int kb) {
-        constexpr int cur = decltype(cur_c)::value, nxt = 1 - cur;
-        const int kn1 = clamp_kb(kb + 1);
-        const bool adv1 = kb + 2 <= kb_last, adv2 = kb + 3 <= kb_last;   // does the next iteration move on a block?
+        constexpr int cur = decltype(cur_c)::value, nxt = (cur + 1) % NS, prv = (cur + NS - 1) % NS;
+        const bool adv1 = kb + NS <= kb_last, adv2 = kb + NS + 1 <= kb_last;   // does the next iteration move on a block?
         const float s_last = s[TM - 1];                    // scale of the previous block's last m-tile (lagged folds)
 #pragma unroll
-        for (int j = 0; j < TM; j++) s[j] = sraw[j] * sb_cur;
+        for (int j = 0; j < TM; j++) s[j] = sraw[j] * sb_raw;
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int t = 0; t < NMFMA; t++) {
@@ -339,23 +355,18 @@ __device__ __forceinline__ void tile_mainloop(
             if (t == BAR_SLOT) {
                 // my DMA loads of the next stage have landed; after the barrier everyone's have, and everyone has
                 // finished reading the current stage (its last fragment was fetched one m-tile ago)
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                // b_scale of the next block was requested in slot 0. Touch it here, where the wait above has
-                // already covered it: the compiler then never waits for it later, behind the DMA loads it
-                // cannot see.
-                asm volatile("" : "+v"(sb_next));
+                wait_for_stage();
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (t == 0) sb_next = SB[(size_t)kn1 * QN + nb + vzero];
             pring[t % PR] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
                 bfrag[i], afrag[j & 1], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
             asm volatile("" : "+v"(pring[t % PR]));          // anchor: the MFMA is issued here, not later
             __builtin_amdgcn_sched_barrier(0);
-            // LDS-DMA: the batch for block kb+1 (started in the previous iteration) continues in the first slots;
-            // the batch for block kb+2 starts right after the barrier
+            // LDS-DMA: the batch for block kb+NS-1 (started in the previous iteration) continues in the first slots;
+            // the batch for block kb+NS starts right after the barrier, into the stage this iteration has consumed
             if (t + TN < NDMA) {
-                issue_dma(t + TN, nxt, dsrc[t + TN]);
+                issue_dma(t + TN, prv, dsrc[t + TN]);
                 dsrc[t + TN] += adv1 ? dma_step(t + TN) : 0;
             }
             if (t >= BAR_SLOT && t - BAR_SLOT < NDMA && t - BAR_SLOT < TN) {
@@ -386,14 +397,19 @@ __device__ __forceinline__ void tile_mainloop(
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        sb_cur = sb_next;
     };
     int kb = kb_begin;
-    for (; kb + 1 < kb_end; kb += 2) {
+    for (; kb + NS - 1 < kb_end; kb += NS) {
         k_block(IntTag<0>{}, kb);
         k_block(IntTag<1>{}, kb + 1);
+        if constexpr (NS > 2) k_block(IntTag<2 % NS>{}, kb + 2);
+        if constexpr (NS > 3) k_block(IntTag<3 % NS>{}, kb + 3);
     }
     if (kb < kb_end) k_block(IntTag<0>{}, kb);
+    if constexpr (NS > 2)
+        if (kb + 1 < kb_end) k_block(IntTag<1>{}, kb + 1);
+    if constexpr (NS > 3)
+        if (kb + 2 < kb_end) k_block(IntTag<2 % NS>{}, kb + 2);
     // folds still owed by the last K block
 #pragma unroll
     for (int t = 0; t < LAG; t++) {
@@ -403,7 +419,6 @@ __device__ __forceinline__ void tile_mainloop(
     }
     // LDS-DMA writes of the last (redundant) prefetches must land before this workgroup's LDS can be handed on
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-
 }
 
 // Stores a wave's accumulators as bf16 into C, masked at the M and N edges. In the MFMA layout a lane owns 4
@@ -521,7 +536,7 @@ __device__ __forceinline__ void exchange_tile_f32(f32x4 (&acc)[BM / WAVES_M / 16
 // Requirements checked by the host: M%16==0, N%16==0, M>=16, N>=16, a/b 16-byte aligned,
 // c 16-byte aligned, K%128==0.
 // ---------------------------------------------------------------------------------------------
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool PARTIAL>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool PARTIAL, int NS = 2>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_tile(
     const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
     const float *__restrict__ SB, void *__restrict__ Cout, int M, int N, int K, int kb_per_split,
@@ -535,7 +550,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
     const int kb_begin = blockIdx.y * kb_per_split;
     const int kb_end = kb_begin + kb_per_split < QK ? kb_begin + kb_per_split : QK;
     f32x4 acc[G::TM][G::TN];
-    tile_mainloop<BM, BN, WAVES_M, WAVES_N>(A, B, SA, SB, M, N, m0, n0, kb_begin, kb_end, lds, acc);
+    tile_mainloop<BM, BN, WAVES_M, WAVES_N, NS>(A, B, SA, SB, M, N, m0, n0, kb_begin, kb_end, lds, acc);
     if constexpr (PARTIAL)
         store_tile_f32<BM, BN, WAVES_M, WAVES_N>(acc, (float *)Cout + ((size_t)blockIdx.y * M + m0) * N + n0, N, M - m0,
                                                  N - n0);
