@@ -251,6 +251,33 @@ def main():
                 print("%-34s %8.2f us %8.1f GB/s (%.1f %% of 8 TB/s; includes the allocation of the outputs by torch)"
                       % (key, u, nbytes / u / 1e3, 100 * nbytes / u / 1e3 / PEAK_HBM_GBS), file=sys.stderr)
                 del src
+        # grouped form (expert GEMMs after sorting tokens by expert): 32 groups of uneven size, N=4096, K=7168
+        rng = np.random.default_rng(1)
+        cuts = np.sort(rng.choice(np.arange(1, 8192 // 16), 31, replace=False)) * 16
+        offs = [0] + [int(x) for x in cuts] + [8192]
+        gm, gn, gk, gg = 8192, 4096, 7168, 32
+        fp8 = torch.float8_e4m3fn
+        ga = torch.randint(0, 120, (gk, gm), dtype=torch.uint8, device="cuda").view(fp8).T
+        gb = torch.randint(0, 120, (gg, gk, gn), dtype=torch.uint8, device="cuda").view(fp8).permute(0, 2, 1)
+        gsa = (torch.rand((gk // 128, gm), device="cuda") * 1e-2).T
+        gsb = (torch.rand((gg, gk // 128, gn // 128), device="cuda") * 1e-2).permute(0, 2, 1)
+        gc = torch.empty((gm, gn), dtype=torch.bfloat16, device="cuda")
+        with torch.cuda.stream(stream):
+            for _ in range(args.warmup // 4 + 5):
+                rfk.fp8_mm_grouped(ga, gb, gsa, gsb, gc, offs)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(50):
+                rfk.fp8_mm_grouped(ga, gb, gsa, gsb, gc, offs)
+            e1.record(stream)
+            stream.synchronize()
+        u = e0.elapsed_time(e1) * 1e3 / 50
+        tf = 2.0 * gm * gn * gk / u / 1e6
+        out["grouped"] = {"workload": "32 groups, %d rows in total (16..%d per group), N=%d K=%d" % (
+                              gm, max(b - a for a, b in zip(offs, offs[1:])), gn, gk),
+                          "us": round(u, 2), "tflops": round(tf, 1), "pct_fp8_mfma_peak": round(100 * tf / PEAK_FP8_TFLOPS, 2)}
+        print("grouped %s: %.2f us  %.1f TFLOP/s (%.1f %% of peak)" % (out["grouped"]["workload"], u, tf,
+              100 * tf / PEAK_FP8_TFLOPS), file=sys.stderr)
     print(json.dumps(out))
     return 0
 

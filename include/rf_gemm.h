@@ -94,6 +94,22 @@ size_t rf_gemm_workspace_bytes(int m, int n, int k);
 int rf_gemm_init(size_t workspace_bytes);
 void rf_gemm_destroy(void);
 
+/* Grouped form: `groups` independent GEMMs sharing N and K in one launch, for expert layers whose tokens have been
+ * sorted by expert. The reference's consumer of such a call is LaunchGroupGEMM(..., h_IDX, ...) over the host array
+ * first_token_offset (src/moe/moe.cpp:204,213-221,244-248; fp16 hipBLASLt there); this is its fp8 block-scaled form.
+ *   a   fp8  [K][M_total]           rows of all groups back to back, M_total = row_offsets[groups]
+ *   as  fp32 [K/128][M_total]
+ *   b   fp8  [groups][K][N]         one weight matrix per group
+ *   bs  fp32 [groups][K/128][ceil(N/128)]
+ *   c   bf16 [M_total][N]
+ *   row_offsets  HOST array of groups+1 ints, row_offsets[0] == 0, non-decreasing; group g owns rows
+ *                row_offsets[g] .. row_offsets[g+1]-1 (empty groups allowed); read before the call returns.
+ * groups <= 256. Offsets that are all multiples of 16 (with N % 16 == 0 and 16-byte aligned a, b, c) take the tiled
+ * kernel in one launch; anything else runs the bounds-checked kernel once per group.
+ * variant: -1 = automatic, else an index into {256x256, 128x256, 128x128, 128x64} tiles. */
+int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const float *bs, void *c, const int *row_offsets,
+                        int groups, int n, int k, int variant, hipStream_t stream);
+
 /* Block quantisers: the step before the GEMM, on the GPU. No counterpart in the reference, whose harness draws
  * fp8 bytes and scales directly (tests/gemm/gemm_test.cpp:64-99); they implement the recipe its callers use:
  * scale = amax/448 over a block (1 if the block is all zero), value = e4m3fn_rne(x / scale).

@@ -115,12 +115,14 @@ struct TileGeom {
 };
 
 // Accumulates into acc the contribution of K blocks [kb_begin, kb_end) to the BM x BN tile at (m0, n0).
+// M is the number of rows of A (and of a_scale) that may be touched, ldm the distance in elements between two
+// K rows of A and of a_scale (ldm == M for a plain GEMM, ldm > M when A is a row range of a larger matrix).
 // All waves of the workgroup call it together. On return every LDS-DMA load has landed, but other waves may still
 // be reading LDS: a barrier is needed before LDS is written again.
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NS = 2>
 __device__ __forceinline__ void tile_mainloop(
     const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
-    const float *__restrict__ SB, int M, int N, int m0, int n0, int kb_begin, int kb_end, uint8_t *lds,
+    const float *__restrict__ SB, int M, int ldm, int N, int m0, int n0, int kb_begin, int kb_end, uint8_t *lds,
     f32x4 (&acc)[BM / WAVES_M / 16][BN / WAVES_N / 16]) {
     using G = TileGeom<BM, BN, WAVES_M, WAVES_N, NS>;
     constexpr int NW = WAVES_M * WAVES_N;
@@ -170,7 +172,7 @@ __device__ __forceinline__ void tile_mainloop(
         int c = (lane % CPR_A) ^ swizzle_of_row<BM>(kl);
         int m = m0 + c * 16;
         if (m + 16 > M) m = M - 16;                           // rows past M: any valid bytes will do
-        goff_a[c_] = (uint32_t)(lane / CPR_A) * (uint32_t)M + (uint32_t)m;
+        goff_a[c_] = (uint32_t)(lane / CPR_A) * (uint32_t)ldm + (uint32_t)m;
     }
 #pragma unroll
     for (int c_ = 0; c_ < NCLS_B; c_++) {
@@ -210,13 +212,13 @@ __device__ __forceinline__ void tile_mainloop(
     const uint32_t lds_dst_a = lds_base + wave * (INST_A * 1024), lds_dst_b = lds_base + OFF_B + wave * (INST_B * 1024),
                    lds_dst_s = lds_base + OFF_S + wave * 256, lds_dst_sb = lds_base + OFF_S + OFF_SB;
     auto dma_src = [&](int d, int kb) -> const uint8_t * {
-        if (d < INST_A) return A + ((size_t)kb * BK + (size_t)(wave * INST_A + d) * RPI_A) * M;
+        if (d < INST_A) return A + ((size_t)kb * BK + (size_t)(wave * INST_A + d) * RPI_A) * ldm;
         if (d < D_SA) return B + ((size_t)kb * BK + (size_t)(wave * INST_B + (d - INST_A)) * RPI_B) * N;
-        if (d == D_SA) return (const uint8_t *)(SA + (size_t)kb * M);
+        if (d == D_SA) return (const uint8_t *)(SA + (size_t)kb * ldm);
         return (const uint8_t *)(SB + (size_t)kb * QN);
     };
     auto dma_step = [&](int d) -> size_t {       // bytes from one K block to the next
-        return d < INST_A ? (size_t)BK * M : d < D_SA ? (size_t)BK * N : d == D_SA ? (size_t)M * 4 : (size_t)QN * 4;
+        return d < INST_A ? (size_t)BK * ldm : d < D_SA ? (size_t)BK * N : d == D_SA ? (size_t)ldm * 4 : (size_t)QN * 4;
     };
     auto issue_dma = [&](int d, int stage, const uint8_t *src) {
         if (d < INST_A) {
@@ -550,7 +552,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
     const int kb_begin = blockIdx.y * kb_per_split;
     const int kb_end = kb_begin + kb_per_split < QK ? kb_begin + kb_per_split : QK;
     f32x4 acc[G::TM][G::TN];
-    tile_mainloop<BM, BN, WAVES_M, WAVES_N, NS>(A, B, SA, SB, M, N, m0, n0, kb_begin, kb_end, lds, acc);
+    tile_mainloop<BM, BN, WAVES_M, WAVES_N, NS>(A, B, SA, SB, M, M, N, m0, n0, kb_begin, kb_end, lds, acc);
     if constexpr (PARTIAL)
         store_tile_f32<BM, BN, WAVES_M, WAVES_N>(acc, (float *)Cout + ((size_t)blockIdx.y * M + m0) * N + n0, N, M - m0,
                                                  N - n0);
@@ -595,7 +597,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_str
         const int m0 = tile_m * BM, n0 = tile_n * BN;
         f32x4 acc[G::TM][G::TN];
         __syncthreads();                     // every wave is done with LDS (previous segment, or the mailbox)
-        tile_mainloop<BM, BN, WAVES_M, WAVES_N>(A, B, SA, SB, M, N, m0, n0, kb0, kb1, lds, acc);
+        tile_mainloop<BM, BN, WAVES_M, WAVES_N>(A, B, SA, SB, M, M, N, m0, n0, kb0, kb1, lds, acc);
         bool write_c = (kb0 == 0 && kb1 == QK);
         if (!write_c) {
             // the host only launches this kernel with T >= P, so a tile has exactly two contributors: the workgroup
@@ -642,13 +644,52 @@ __global__ __launch_bounds__(256) void reduce_splitk_bf16(const float *__restric
 }
 
 // ---------------------------------------------------------------------------------------------
+// Grouped form: `groups` independent GEMMs that share N and K, one launch. A (and a_scale, C) hold the rows of all
+// groups back to back (group g owns rows row_start[g] .. row_start[g+1]-1 of an M_total-row matrix), B and b_scale
+// hold one [K][N] / [K/128][QN] block per group. This is the layout of expert GEMMs after tokens have been sorted by
+// expert (the reference's consumer is LaunchGroupGEMM over first_token_offset, src/moe/moe.cpp:213-248, which runs
+// fp16 hipBLASLt there). One workgroup per (group, tile): the table is small enough to travel as a kernel argument.
+// Requirements checked by the host: every row_start a multiple of 16 (and so M_total), N % 16 == 0, K % 128 == 0.
+// ---------------------------------------------------------------------------------------------
+constexpr int kMaxGroups = 256;
+struct GroupTable {
+    int row_start[kMaxGroups + 1];      // prefix of rows
+    int tile_start[kMaxGroups + 1];     // prefix of workgroups
+};
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_grouped(
+    const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
+    const float *__restrict__ SB, uint16_t *__restrict__ C, int M_total, int N, int K, int groups, int tiles_n,
+    int group_m, const GroupTable table) {
+    using G = TileGeom<BM, BN, WAVES_M, WAVES_N>;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    // group of this workgroup: the last g with tile_start[g] <= blockIdx.x (empty groups own no workgroup)
+    int lo = 0, hi = groups;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (table.tile_start[mid] <= (int)blockIdx.x) lo = mid; else hi = mid;
+    }
+    const int grp = lo, row0 = table.row_start[grp], rows = table.row_start[grp + 1] - row0;
+    const int local = blockIdx.x - table.tile_start[grp];
+    const int tiles_m = (rows + BM - 1) / BM;
+    int tile_m, tile_n;
+    tile_of_block(local, tiles_m * tiles_n, tiles_m, tiles_n, group_m, false, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int QK = K / BK, QN = (N + 127) / 128;
+    f32x4 acc[G::TM][G::TN];
+    tile_mainloop<BM, BN, WAVES_M, WAVES_N>(A + row0, B + (size_t)grp * K * N, SA + row0, SB + (size_t)grp * QK * QN,
+                                            rows, M_total, N, m0, n0, 0, QK, lds, acc);
+    store_tile_bf16<BM, BN, WAVES_M, WAVES_N>(acc, C + (size_t)row0 * N, rows, N, m0, n0, lds);
+}
+
+// ---------------------------------------------------------------------------------------------
 // Bounds-checked kernel for shapes or alignments the tiled kernel does not take (M or N not a
 // multiple of 16, unaligned pointers). One wave per 16x16 output tile, bytes gathered directly
 // from global memory; out-of-range rows/columns contribute zeros and are not stored.
 // ---------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(64) void gemm_fp8_blockscale_checked(
     const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
-    const float *__restrict__ SB, uint16_t *__restrict__ C, int M, int N, int K) {
+    const float *__restrict__ SB, uint16_t *__restrict__ C, int M, int ldm, int N, int K) {
     const int lane = threadIdx.x, L = lane & 15, g = lane >> 4;
     const int m0 = blockIdx.y * 16, n0 = blockIdx.x * 16;
     const int QK = K / BK, QN = (N + 127) / 128;
@@ -660,12 +701,12 @@ __global__ __launch_bounds__(64) void gemm_fp8_blockscale_checked(
 #pragma unroll
         for (int j = 0; j < 32; j++) {
             size_t k = (size_t)kb * BK + 32 * g + j;
-            fa.b[j] = m_ok ? A[k * M + m_ld] : (uint8_t)0;
+            fa.b[j] = m_ok ? A[k * ldm + m_ld] : (uint8_t)0;
             fb.b[j] = n_ok ? B[k * N + n_ld] : (uint8_t)0;
         }
         f32x4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb.v, fa.v, (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
         // lane holds D[n = n0+4g+e][m = m0+L]
-        float sa = m_ok ? SA[(size_t)kb * M + m_ld] : 0.f;
+        float sa = m_ok ? SA[(size_t)kb * ldm + m_ld] : 0.f;
 #pragma unroll
         for (int e = 0; e < 4; e++) {
             int n = n0 + 4 * g + e;

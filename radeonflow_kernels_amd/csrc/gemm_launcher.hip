@@ -245,7 +245,7 @@ int launch(const void *a, const void *b, const float *as, const float *bs, void 
     if (cfg.variant < 0) {
         dim3 grid(ceil_div(n, 16), ceil_div(m, 16));
         hipLaunchKernelGGL(rf::gemm_fp8_blockscale_checked, grid, dim3(64), 0, stream, (const uint8_t *)a,
-                           (const uint8_t *)b, as, bs, (uint16_t *)c, m, n, k);
+                           (const uint8_t *)b, as, bs, (uint16_t *)c, m, m, n, k);
         RF_HIP(hipGetLastError());
         return RF_OK;
     }
@@ -435,7 +435,95 @@ int launch_quantize(const void *x, int rows, int k, void *out, float *scales, hi
 }
 }  // namespace
 
+namespace {
+typedef void (*grouped_kernel_t)(const uint8_t *, const uint8_t *, const float *, const float *, uint16_t *, int, int, int,
+                                 int, int, int, const rf::GroupTable);
+struct GroupedVariant {
+    int bm, bn, threads, lds;
+    grouped_kernel_t kernel;
+};
+#define RF_GROUPED(BM, BN, WM, WN) \
+    GroupedVariant { BM, BN, WM *WN * 64, rf::TileGeom<BM, BN, WM, WN>::LDS_BYTES, rf::gemm_fp8_blockscale_grouped<BM, BN, WM, WN> }
+const GroupedVariant kGroupedVariants[] = {RF_GROUPED(256, 256, 2, 4), RF_GROUPED(128, 256, 2, 4), RF_GROUPED(128, 128, 2, 2),
+                                           RF_GROUPED(128, 64, 2, 1)};
+constexpr int kNumGroupedVariants = sizeof(kGroupedVariants) / sizeof(kGroupedVariants[0]);
+bool g_grouped_attrs_set = false;
+
+long grouped_tiles(const GroupedVariant &v, const int *row_offsets, int groups, int n) {
+    long t = 0;
+    for (int g = 0; g < groups; g++) t += (long)ceil_div(row_offsets[g + 1] - row_offsets[g], v.bm) * ceil_div(n, v.bn);
+    return t;
+}
+}  // namespace
+
 extern "C" {
+
+int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const float *bs, void *c, const int *row_offsets,
+                        int groups, int n, int k, int variant, hipStream_t stream) {
+    g_last_error.clear();
+    if (!row_offsets) return fail(RF_ERR_NULL_POINTER, "row_offsets is null");
+    if (groups < 1 || groups > rf::kMaxGroups)
+        return fail(RF_ERR_BAD_SHAPE, "groups must be between 1 and " + std::to_string(rf::kMaxGroups));
+    if (n < 1 || k < rf::BK || k % rf::BK != 0 || row_offsets[0] != 0)
+        return fail(RF_ERR_BAD_SHAPE, "unsupported shape (need N>=1, K a positive multiple of 128, row_offsets[0] == 0)");
+    for (int g = 0; g < groups; g++)
+        if (row_offsets[g + 1] < row_offsets[g]) return fail(RF_ERR_BAD_SHAPE, "row_offsets must not decrease");
+    const int m_total = row_offsets[groups];
+    if (m_total == 0) return RF_OK;
+    if (!a || !b || !as || !bs || !c) return fail(RF_ERR_NULL_POINTER, "null device pointer");
+    if (variant >= kNumGroupedVariants || variant < -1) return fail(RF_ERR_BAD_CONFIG, "no such grouped variant");
+    State &s = state();
+    std::lock_guard<std::mutex> lock(s.mu);
+    int rc = ensure_device_info(s);
+    if (rc != RF_OK) return rc;
+    if (!g_grouped_attrs_set) {
+        for (const GroupedVariant &v : kGroupedVariants)
+            RF_HIP(hipFuncSetAttribute((const void *)v.kernel, hipFuncAttributeMaxDynamicSharedMemorySize, v.lds));
+        g_grouped_attrs_set = true;
+    }
+    const int qk = k / rf::BK, qn = ceil_div(n, 128);
+    bool tiled = n % 16 == 0 && ((uintptr_t)a % 16) == 0 && ((uintptr_t)b % 16) == 0 && ((uintptr_t)c % 16) == 0;
+    for (int g = 0; g <= groups && tiled; g++) tiled = row_offsets[g] % 16 == 0;
+    if (!tiled) {
+        // ragged groups or unaligned operands: the bounds-checked kernel, one launch per non-empty group
+        for (int g = 0; g < groups; g++) {
+            const int r0 = row_offsets[g], rows = row_offsets[g + 1] - r0;
+            if (rows == 0) continue;
+            dim3 grid(ceil_div(n, 16), ceil_div(rows, 16));
+            hipLaunchKernelGGL(rf::gemm_fp8_blockscale_checked, grid, dim3(64), 0, stream, (const uint8_t *)a + r0,
+                               (const uint8_t *)b + (size_t)g * k * n, as + r0, bs + (size_t)g * qk * qn,
+                               (uint16_t *)c + (size_t)r0 * n, rows, m_total, n, k);
+            RF_HIP(hipGetLastError());
+        }
+        return RF_OK;
+    }
+    if (variant < 0) {
+        // the largest tile that still gives every CU a workgroup; failing that, the one with the most workgroups
+        variant = kNumGroupedVariants - 1;
+        for (int v = 0; v < kNumGroupedVariants; v++)
+            if (grouped_tiles(kGroupedVariants[v], row_offsets, groups, n) >= s.num_cu) {
+                variant = v;
+                break;
+            }
+    }
+    const GroupedVariant &v = kGroupedVariants[variant];
+    rf::GroupTable table;
+    const int tiles_n = ceil_div(n, v.bn);
+    int tiles = 0;
+    for (int g = 0; g < groups; g++) {
+        table.row_start[g] = row_offsets[g];
+        table.tile_start[g] = tiles;
+        tiles += ceil_div(row_offsets[g + 1] - row_offsets[g], v.bm) * tiles_n;
+    }
+    for (int g = groups; g <= rf::kMaxGroups; g++) {
+        table.row_start[g] = m_total;
+        table.tile_start[g] = tiles;
+    }
+    hipLaunchKernelGGL(v.kernel, dim3(tiles), dim3(v.threads), v.lds, stream, (const uint8_t *)a, (const uint8_t *)b, as,
+                       bs, (uint16_t *)c, m_total, n, k, groups, tiles_n, 8, table);
+    RF_HIP(hipGetLastError());
+    return RF_OK;
+}
 
 int rf_quantize_a_f32(const float *x, int m, int k, void *a, float *as, hipStream_t stream) {
     return launch_quantize<true, false>(x, m, k, a, as, stream);

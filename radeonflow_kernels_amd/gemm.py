@@ -39,7 +39,7 @@ class PerfMetrics(ctypes.Structure):
 
 EXPORTS = ("run", "rf_fp8_gemm", "rf_fp8_gemm_ex", "rf_gemm_select_config", "rf_gemm_num_variants",
            "rf_gemm_variant_info", "rf_gemm_variant_has_stream_k", "rf_gemm_variant_has_persistent", "rf_gemm_workspace_bytes", "rf_gemm_init", "rf_gemm_destroy",
-           "rf_gemm_last_error", "rf_quantize_a_f32", "rf_quantize_a_bf16", "rf_quantize_b_f32", "rf_quantize_b_bf16")
+           "rf_gemm_last_error", "rf_fp8_gemm_grouped", "rf_quantize_a_f32", "rf_quantize_a_bf16", "rf_quantize_b_f32", "rf_quantize_b_bf16")
 
 
 def lib():
@@ -72,6 +72,8 @@ def lib():
         L.rf_gemm_init.restype = i32
         L.rf_gemm_destroy.restype = None
         L.rf_gemm_last_error.restype = ctypes.c_char_p
+        L.rf_fp8_gemm_grouped.argtypes = [ctypes.c_void_p] * 5 + [ctypes.POINTER(i32), i32, i32, i32, i32, ctypes.c_void_p]
+        L.rf_fp8_gemm_grouped.restype = i32
         for name in ("rf_quantize_a_f32", "rf_quantize_a_bf16", "rf_quantize_b_f32", "rf_quantize_b_bf16"):
             f = getattr(L, name)
             f.argtypes = [ctypes.c_void_p, i32, i32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
@@ -116,6 +118,33 @@ def fp8_mm(a, b, a_scale, b_scale, c, config=None):
                               m, n, k, cfg, stream)
     if rc != RF_OK:
         raise RuntimeError("rf_fp8_gemm failed (%d): %s" % (rc, last_error()))
+
+
+def fp8_mm_grouped(a, b, a_scale, b_scale, c, row_offsets, variant=-1):
+    """Grouped GEMM: rows row_offsets[g]..row_offsets[g+1]-1 of a / a_scale / c belong to group g and are multiplied
+    with b[g], b_scale[g].
+      a [M_total, K] fp8 stride (1, M_total); a_scale [M_total, K/128] fp32 stride (1, M_total);
+      b [G, N, K] fp8 stride (K*N, 1, N); b_scale [G, ceil(N/128), K/128] fp32 stride (QK*QN, 1, QN);
+      c [M_total, N] bf16 contiguous; row_offsets: sequence of G+1 ints on the host."""
+    m_total, k = a.shape
+    groups, n, _ = b.shape
+    qk, qn = k // 128, (n + 127) // 128
+    ok = (a.dtype == torch.float8_e4m3fn and b.dtype == torch.float8_e4m3fn and c.dtype == torch.bfloat16
+          and a_scale.dtype == torch.float32 and b_scale.dtype == torch.float32
+          and tuple(b.shape) == (groups, n, k) and tuple(c.shape) == (m_total, n) and c.is_contiguous()
+          and (m_total <= 1 or k == 1 or a.stride() == (1, m_total)) and tuple(a_scale.shape) == (m_total, qk)
+          and (m_total <= 1 or qk == 1 or a_scale.stride() == (1, m_total))
+          and b.stride() == (k * n, 1, n) and tuple(b_scale.shape) == (groups, qn, qk)
+          and (b_scale.stride() == (qk * qn, 1, qn) or qn == 1 or qk == 1) and len(row_offsets) == groups + 1)
+    if not ok:
+        raise ValueError("fp8_mm_grouped: operands do not have the documented dtypes / shapes / strides")
+    offs = (ctypes.c_int32 * (groups + 1))(*[int(x) for x in row_offsets])
+    stream = ctypes.c_void_p(torch.cuda.current_stream(a.device).cuda_stream)
+    with torch.cuda.device(a.device):
+        rc = lib().rf_fp8_gemm_grouped(a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(), c.data_ptr(),
+                                       offs, groups, n, k, variant, stream)
+    if rc != RF_OK:
+        raise RuntimeError("rf_fp8_gemm_grouped failed (%d): %s" % (rc, last_error()))
 
 
 def custom_kernel(data):

@@ -25,6 +25,38 @@ def test_library_exports_every_declared_symbol():
     assert sorted(gemm.EXPORTS) == names
 
 
+def _declared_parameter_counts():
+    text = open(os.path.join(ROOT, "include", "rf_gemm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    out = {}
+    for name, params in re.findall(r"\b(run|rf_[a-z0-9_]+)\s*\(([^)]*)\)\s*;", text):
+        params = params.strip()
+        out[name] = 0 if params in ("", "void") else params.count(",") + 1
+    return out
+
+
+def test_python_binding_declares_as_many_arguments_as_the_header():
+    """A ctypes prototype with the wrong number or kind of arguments silently truncates 64-bit device pointers to
+    32 bits: every entry point the mirror calls with pointers must carry argtypes of the header's length, and
+    every pointer parameter must be a pointer type."""
+    from radeonflow_kernels_amd import gemm
+    L = gemm.lib()
+    counts = _declared_parameter_counts()
+    with_pointers = [n for n in counts if n not in ("rf_gemm_num_variants", "rf_gemm_destroy", "rf_gemm_last_error")]
+    for name in with_pointers:
+        at = getattr(L, name).argtypes
+        assert at is not None, "%s has no ctypes prototype" % name
+        assert len(at) == counts[name], "%s: %d argtypes, header declares %d" % (name, len(at), counts[name])
+    text = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "rf_gemm.h")).read(), flags=re.S)
+    for name, params in re.findall(r"\b(run|rf_[a-z0-9_]+)\s*\(([^)]*)\)\s*;", text):
+        if name not in with_pointers:
+            continue
+        for decl, ct in zip(params.split(","), getattr(L, name).argtypes):
+            is_ptr = "*" in decl or "hipStream_t" in decl
+            ct_ptr = ct is ctypes.c_void_p or ct is ctypes.c_char_p or hasattr(ct, "contents")
+            assert is_ptr == ct_ptr, "%s: parameter '%s' bound as %r" % (name, decl.strip(), ct)
+
+
 def test_perf_metrics_layout_matches_the_reference_struct():
     from radeonflow_kernels_amd.gemm import PerfMetrics, PerfMetricEntry, GemmConfig
     assert ctypes.sizeof(PerfMetricEntry) == 28

@@ -1,0 +1,117 @@
+"""Grouped GEMM (one launch, rows sorted by group, one weight matrix per group) against the oracle applied group
+by group. Exact data for bit-for-bit equality, quantised N(0,1) data at the graded tolerance."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import cref, ref_kernel as rk
+from helpers import RTOL, ATOL, assert_close_to_oracle, bf16_bits, exact_problem, oracle_bf16
+
+pytestmark = pytest.mark.gpu
+CANARY = 2048
+
+
+@pytest.fixture(scope="module")
+def rfk():
+    import radeonflow_kernels_amd as m
+    m.lib()
+    return m
+
+
+def _grouped_problem(rows, n, k, seed, exact):
+    """Per-group problems from the usual generators, glued into the grouped layouts.
+    Returns (device tensors a, b, a_scale, b_scale, c, canary buffer), row_offsets, expected bf16 bits [M_total, N]."""
+    offs = np.concatenate([[0], np.cumsum(rows)]).astype(np.int64)
+    m_total, groups = int(offs[-1]), len(rows)
+    qk, qn = k // 128, (n + 127) // 128
+    a_km = np.zeros((k, m_total), np.uint8)
+    as_qm = np.zeros((qk, m_total), np.float32)
+    b_gkn = np.zeros((groups, k, n), np.uint8)
+    bs_gqq = np.zeros((groups, qk, qn), np.float32)
+    exp = np.zeros((m_total, n), np.uint16)
+    for g, r in enumerate(rows):
+        mg = max(int(r), 16)            # empty groups still get weights
+        data = exact_problem(mg, n, k, seed + g) if exact else rk.generate_input_blockquant(mg, n, k, seed + g)
+        a, b, sa, sb = rk.raw_layouts(data)
+        b_gkn[g], bs_gqq[g] = b, sb
+        if r:
+            a_km[:, offs[g]:offs[g + 1]] = a[:, :r]
+            as_qm[:, offs[g]:offs[g + 1]] = sa[:, :r]
+            sub = (data[0][:r], data[1], data[2][:r], data[3], torch.zeros((int(r), n), dtype=torch.bfloat16))
+            exp[offs[g]:offs[g + 1]] = oracle_bf16(sub)
+    dev, fp8 = torch.device("cuda:0"), torch.float8_e4m3fn
+    a_t = torch.from_numpy(a_km).to(dev).view(fp8).T                       # [M_total, K] stride (1, M_total)
+    as_t = torch.from_numpy(as_qm).to(dev).T
+    b_t = torch.from_numpy(b_gkn).to(dev).view(fp8).permute(0, 2, 1)       # [G, N, K] stride (K*N, 1, N)
+    bs_t = torch.from_numpy(bs_gqq).to(dev).permute(0, 2, 1)
+    buf = torch.full((m_total * n + CANARY,), -7.0, dtype=torch.bfloat16, device=dev)
+    c = buf[: m_total * n].view(m_total, n)
+    c.zero_()
+    return (a_t, b_t, as_t, bs_t, c, buf), [int(x) for x in offs], exp
+
+
+def _check_canary(buf, used):
+    assert np.all(buf[used:].float().cpu().numpy() == -7.0), "store past the end of C"
+
+
+CASES = [([256, 128, 512, 64], 512, 256), ([16, 0, 48, 400, 0, 32], 576, 384), ([1024], 256, 512),
+         ([128] * 32, 2048, 256), ([0, 0, 272], 144, 128), ([640, 16, 16, 2048, 112], 7168, 256)]
+
+
+@pytest.mark.parametrize("rows,n,k", CASES)
+def test_grouped_bit_exact_on_exact_data(rfk, rows, n, k):
+    g, offs, exp = _grouped_problem(rows, n, k, seed=11 * n + k, exact=True)
+    for variant in (-1, 0, 1, 2, 3):
+        g[4].zero_()
+        rfk.fp8_mm_grouped(*g[:5], offs, variant=variant)
+        torch.cuda.synchronize()
+        assert np.array_equal(bf16_bits(g[4]), exp), "variant %d" % variant
+        _check_canary(g[5], g[4].numel())
+
+
+@pytest.mark.parametrize("rows,n,k", [([256, 128, 512, 64], 512, 1024), ([48, 400, 32], 576, 7168)])
+def test_grouped_quantised_data_within_tolerance(rfk, rows, n, k):
+    g, offs, exp = _grouped_problem(rows, n, k, seed=5, exact=False)
+    rfk.fp8_mm_grouped(*g[:5], offs)
+    torch.cuda.synchronize()
+    assert_close_to_oracle(g[4], exp, RTOL, ATOL, "grouped")
+    _check_canary(g[5], g[4].numel())
+
+
+@pytest.mark.parametrize("rows,n,k", [([5, 17, 0, 100], 130, 256), ([33, 64], 72, 128)])
+def test_grouped_ragged_groups_take_the_checked_kernel(rfk, rows, n, k):
+    g, offs, exp = _grouped_problem(rows, n, k, seed=3, exact=True)
+    rfk.fp8_mm_grouped(*g[:5], offs)
+    torch.cuda.synchronize()
+    assert np.array_equal(bf16_bits(g[4]), exp)
+    _check_canary(g[5], g[4].numel())
+
+
+def test_grouped_equals_separate_gemms(rfk):
+    """The grouped launch and one plain fp8_mm per group give the same bits (same kernel family, same order)."""
+    rows, n, k = [256, 384, 128], 1536, 1024
+    g, offs, _ = _grouped_problem(rows, n, k, seed=9, exact=False)
+    rfk.fp8_mm_grouped(*g[:5], offs, variant=1)
+    torch.cuda.synchronize()
+    a, b, sa, sb, c = g[:5]
+    for i, r in enumerate(rows):
+        lo, hi = offs[i], offs[i + 1]
+        ai = a[lo:hi].T.contiguous().T                # standalone [r, K] with stride (1, r)
+        si = sa[lo:hi].T.contiguous().T
+        ci = torch.zeros((r, n), dtype=torch.bfloat16, device=a.device)
+        rfk.fp8_mm(ai, b[i], si, sb[i], ci, config=rfk.GemmConfig(3, 1, 8, 0))      # 128x256 tiles, like variant 1
+        torch.cuda.synchronize()
+        assert torch.equal(ci.view(torch.uint16), c[lo:hi].view(torch.uint16)), "group %d" % i
+
+
+def test_grouped_status_codes(rfk):
+    import ctypes
+    L = rfk.lib()
+    offs = (ctypes.c_int32 * 3)(0, 16, 8)
+    assert L.rf_fp8_gemm_grouped(None, None, None, None, None, offs, 2, 128, 128, -1, None) == 1      # decreasing offsets
+    offs = (ctypes.c_int32 * 2)(0, 0)
+    assert L.rf_fp8_gemm_grouped(None, None, None, None, None, offs, 1, 128, 128, -1, None) == 0      # nothing to do
+    offs = (ctypes.c_int32 * 2)(0, 16)
+    assert L.rf_fp8_gemm_grouped(None, None, None, None, None, offs, 1, 128, 128, -1, None) == 2      # null pointers
+    assert L.rf_fp8_gemm_grouped(None, None, None, None, None, offs, 1, 128, 100, -1, None) == 1      # bad K
+    assert L.rf_fp8_gemm_grouped(None, None, None, None, None, offs, 300, 128, 128, -1, None) == 1    # too many groups
