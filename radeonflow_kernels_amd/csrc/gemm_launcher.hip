@@ -258,8 +258,13 @@ int launch(const void *a, const void *b, const float *as, const float *bs, void 
     dim3 grid(tiles_m * tiles_n, splits);
     dim3 block(v.threads());
     if (cfg.stream_k == RF_SCHEDULE_PERSISTENT) {
+        // as many resident workgroups as the LDS of a CU holds (small tiles: two or three per CU, so that one's
+        // store drain overlaps another's compute)
         const int T = tiles_m * tiles_n;
-        hipLaunchKernelGGL(v.persistent, dim3(T < s.num_cu ? T : s.num_cu), block, v.lds_persistent, stream,
+        int per_cu = (160 * 1024) / v.lds_persistent;
+        if (per_cu > 2048 / v.threads()) per_cu = 2048 / v.threads();
+        const int P = s.num_cu * (per_cu < 1 ? 1 : per_cu);
+        hipLaunchKernelGGL(v.persistent, dim3(T < P ? T : P), block, v.lds_persistent, stream,
                            (const uint8_t *)a, (const uint8_t *)b, as, bs, (uint16_t *)c, m, n, k, tiles_m, tiles_n,
                            cfg.group_m);
         RF_HIP(hipGetLastError());
