@@ -133,7 +133,7 @@ __device__ __forceinline__ void tile_mainloop(
     // of any stage is "per-lane base register + immediate": no address arithmetic in the loop.
     constexpr int STAGE_A = G::STAGE_A, STAGE_B = G::STAGE_B, STAGE_S = G::STAGE_S;
     constexpr int OFF_B = NS * STAGE_A, OFF_S = NS * (STAGE_A + STAGE_B), OFF_SB = BM * 4;   // OFF_SB inside an S region
-    static_assert(NS >= 2 && NS <= 4, "two to four stages");
+    static_assert(NS == 2, "more than two stages would need vmcnt(n > 0) waits, which LDS-DMA loads do not support safely");
     constexpr int INST_A = STAGE_A / 1024 / NW, INST_B = STAGE_B / 1024 / NW;   // 1 KiB per wave instruction
     constexpr int NSC = BM / 64;                                                // scale loads: 64 floats each
     static_assert(STAGE_A % (1024 * NW) == 0 && STAGE_B % (1024 * NW) == 0, "loads must divide evenly over waves");
@@ -239,13 +239,10 @@ __device__ __forceinline__ void tile_mainloop(
                          :: "v"(goff_sb), "s"(src), "s"(lds_dst_sb), "n"(stage * STAGE_S) : "memory", "scc");
         }
     };
-    // Wait until the loads of every K block except the newest NS-2 have landed. vmcnt counts this wave's loads in
-    // issue order; the optional scale loads are left out of the allowance, which errs on the side of waiting.
-    auto wait_for_stage = [&]() {
-        if constexpr (NS == 2) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(%0)" :: "n"((NS - 2) * (INST_A + INST_B)) : "memory");
-    };
-    static_assert((NS - 2) * (INST_A + INST_B) < 64, "vmcnt is a 6-bit counter");
+    // Wait until every load this wave has issued has landed. Only vmcnt(0) is used: with LDS-DMA loads a wait for
+    // "all but the newest n" is not safe (a later load that hits in L2 was seen to complete before an earlier one
+    // that missed), which is also why the kernel has exactly two stages.
+    auto wait_for_stage = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
 
     // ---- LDS -> MFMA operands: per-lane byte offsets of the transpose reads (stage 0, t = 0) ----
     // lane (L,g) of read t points at row k = 32g + 8t + L/2, half (L&1) of 16-byte chunk c.

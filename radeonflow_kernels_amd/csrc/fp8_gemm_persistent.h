@@ -35,8 +35,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
     using P = PersistentGeom<BM, BN, WAVES_M, WAVES_N>;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     constexpr int NW = G::NW, WM = G::WM, WN = G::WN, TM = G::TM, TN = G::TN;
-    constexpr int STAGE_A = BK * BM, STAGE_B = BK * BN, STAGE_S = BM * 4;
-    constexpr int OFF_B = 2 * STAGE_A, OFF_S = 2 * STAGE_A + 2 * STAGE_B;
+    constexpr int STAGE_A = G::STAGE_A, STAGE_B = G::STAGE_B, STAGE_S = G::STAGE_S;
+    constexpr int OFF_B = 2 * STAGE_A, OFF_S = 2 * STAGE_A + 2 * STAGE_B, OFF_SB = BM * 4;
     static_assert(STAGE_A + 3 * 8 * BM + 16 * (BM / 16) < 65536 && STAGE_B + 3 * 8 * BN + 16 * (BN / 16) < 65536,
                   "stage offsets must fit the immediate offset of an LDS read");
     constexpr int INST_A = STAGE_A / 1024 / NW, INST_B = STAGE_B / 1024 / NW;
@@ -75,7 +75,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
     auto rep_a = [](int c) { return c % PER_A + (c / PER_A) * (32 / RPI_A); };
     auto cls_b = [](int i) { return i % PER_B + PER_B * (i * RPI_B / 32); };
     auto rep_b = [](int c) { return c % PER_B + (c / PER_B) * (32 / RPI_B); };
-    uint32_t goff_a[NCLS_A], goff_b[NCLS_B], goff_s;
+    uint32_t goff_a[NCLS_A], goff_b[NCLS_B], goff_s, goff_sb;
 #pragma unroll
     for (int c_ = 0; c_ < NCLS_A; c_++) {
         const int kl = (wave * INST_A + rep_a(c_)) * RPI_A + lane / CPR_A;
@@ -91,34 +91,46 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
     {
         const int sl = (wave < NSC ? wave : 0) * 64 + lane, r = sl % WM;
         goff_s = (uint32_t)((sl / WM) * WM + 16 * (r % TM) + r / TM) * 4u;
+        // b_scale slots: the tile's column blocks (N is a multiple of BN here, so they all exist); the other lanes
+        // repeat the last one
+        constexpr int NBLK = BN / 128 > 0 ? BN / 128 : 1;
+        goff_sb = (uint32_t)(lane < NBLK ? lane : NBLK - 1) * 4u;
     }
     const uint32_t lds_base = (uint32_t)(uintptr_t)(RF_LDS uint8_t *)lds;
-    constexpr int NDMA = INST_A + INST_B + 1;
+    constexpr int D_SA = INST_A + INST_B, D_SB = D_SA + 1, NDMA = D_SB + 1;
     const uint32_t lds_dst_a = lds_base + wave * (INST_A * 1024), lds_dst_b = lds_base + OFF_B + wave * (INST_B * 1024),
-                   lds_dst_s = lds_base + OFF_S + wave * 256;
+                   lds_dst_s = lds_base + OFF_S + wave * 256, lds_dst_sb = lds_base + OFF_S + OFF_SB;
     auto dma_src = [&](int d, int m0, int n0, int kb) -> const uint8_t * {
         if (d < INST_A) return A + ((size_t)kb * BK + (size_t)(wave * INST_A + d) * RPI_A) * M + m0;
-        if (d < INST_A + INST_B) return B + ((size_t)kb * BK + (size_t)(wave * INST_B + (d - INST_A)) * RPI_B) * N + n0;
-        return (const uint8_t *)(SA + (size_t)kb * M + m0);
+        if (d < D_SA) return B + ((size_t)kb * BK + (size_t)(wave * INST_B + (d - INST_A)) * RPI_B) * N + n0;
+        if (d == D_SA) return (const uint8_t *)(SA + (size_t)kb * M + m0);
+        return (const uint8_t *)(SB + (size_t)kb * QN + (n0 >> 7));
     };
     auto dma_step = [&](int d) -> size_t {
-        return d < INST_A ? (size_t)BK * M : d < INST_A + INST_B ? (size_t)BK * N : (size_t)M * 4;
+        return d < INST_A ? (size_t)BK * M : d < D_SA ? (size_t)BK * N : d == D_SA ? (size_t)M * 4 : (size_t)QN * 4;
     };
     auto issue_dma = [&](int d, int stage, const uint8_t *src) {
         if (d < INST_A) {
             asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                          :: "v"(goff_a[cls_a(d < INST_A ? d : 0)]), "s"(src), "s"(lds_dst_a), "n"(d * 1024 + stage * STAGE_A)
                          : "memory", "scc");
-        } else if (d < INST_A + INST_B) {
+        } else if (d < D_SA) {
             const int e = d - INST_A < INST_B ? d - INST_A : 0;
             asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                          :: "v"(goff_b[cls_b(e >= 0 ? e : 0)]), "s"(src), "s"(lds_dst_b), "n"(e * 1024 + stage * STAGE_B)
                          : "memory", "scc");
-        } else if (wave < NSC) {
+        } else if (d == D_SA) {
+            if (wave < NSC)
+                asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+                             :: "v"(goff_s), "s"(src), "s"(lds_dst_s), "n"(stage * STAGE_S) : "memory", "scc");
+        } else if (wave == 0) {
             asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
-                         :: "v"(goff_s), "s"(src), "s"(lds_dst_s), "n"(stage * STAGE_S) : "memory", "scc");
+                         :: "v"(goff_sb), "s"(src), "s"(lds_dst_sb), "n"(stage * STAGE_S) : "memory", "scc");
         }
     };
+    // The wait before the barrier is always vmcnt(0). Waiting for "all but the newest n loads" is not safe with
+    // LDS-DMA loads: a later load that hits in L2 was seen to complete before an earlier one that missed.
+    auto wait_for_stage = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
 
     // ---- LDS -> MFMA operands (see tile_mainloop) ----
     const int krow = 32 * g + (L >> 1);
@@ -126,9 +138,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
     const uint32_t aoff_base = krow * BM + (((wm * TM) ^ swizzle_of_row<BM>(krow)) << 4) + 8 * (L & 1);
     const uint32_t boff_base = OFF_B + krow * BN + (((wn * TN) ^ swizzle_of_row<BN>(krow)) << 4) + 8 * (L & 1);
     const uint32_t soff = OFF_S + (wm * WM + L * TM) * 4;
-
-    int vzero;
-    asm volatile("v_mov_b32 %0, 0" : "=v"(vzero));
+    const uint32_t sboff = OFF_S + OFF_SB + (((wn * WN) >> 7) << 2);    // n0 is a multiple of BN: block inside the tile
 
     constexpr int PR = 4, LAG = 3, NMFMA = TM * TN, BAR_SLOT = (TM - 1) * TN;
     static_assert(LAG < TN && LAG < PR && TM % 2 == 0 && NDMA - TN <= BAR_SLOT, "same schedule as tile_mainloop");
@@ -136,7 +146,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
     f32x4 acc[TM][TN];
     i32x8 bfrag[TN], afrag[2];
     f32x4 pring[PR];
-    float s[TM], sraw[TM], sb_cur = 0.f, sb_next = 0.f;
+    float s[TM], sraw[TM], sb_raw = 0.f;
 #pragma unroll
     for (int j = 0; j < TM; j++)
 #pragma unroll
@@ -172,36 +182,33 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
 #pragma unroll
             for (int e = 0; e < 4; e++) sraw[4 * q + e] = v[e];
         }
+        sb_raw = *(RF_LDS float *)(lds + stage * STAGE_S + sboff);
     };
 
     // ---- two load cursors run ahead of the compute position ----
-    // cursor 1 = the K block after the current one (DMA instructions d >= TN, issued in the first slots of a step, and
-    // the b_scale load); cursor 2 = two blocks ahead (instructions d < TN, issued after the barrier). Each holds its
-    // tile ordinal, K block and the running source pointers of its instructions; crossing into the next tile
-    // recomputes the pointers from that tile's origin.
+    // cursor 1 = the K block after the current one (DMA instructions d >= TN, issued in the first slots of a step);
+    // cursor 2 = two blocks ahead (instructions d < TN, issued after the barrier). Each holds its tile ordinal, K block
+    // and the running source pointers of its instructions; crossing into the next tile recomputes the pointers from
+    // that tile's origin.
     const uint8_t *dsrc[NDMA];
     int c1_r = 0, c1_kb = 0, c2_r = 0, c2_kb = 0;     // set below
-    int sb_off1 = 0;                                  // index into SB of cursor 1's block for this wave's columns
-    auto nb_of = [&](int n0) { return (n0 + wn * WN) >> 7; };
-    auto seek = [&](bool first_group, int r, int kb) {   // point a cursor's instructions at (tile r, block kb)
+    auto seek = [&](int which, int r, int kb) {        // point a cursor's instructions at (tile r, block kb)
         int m0, n0;
         tile_origin(r, m0, n0);
 #pragma unroll
         for (int d = 0; d < NDMA; d++)
-            if ((d >= TN) == first_group) dsrc[d] = dma_src(d, m0, n0, kb);
-        if (first_group) sb_off1 = kb * QN + nb_of(n0);
+            if ((d >= TN) == (which == 1)) dsrc[d] = dma_src(d, m0, n0, kb);
     };
-    auto advance = [&](bool first_group, int &r, int &kb) {   // move a cursor one K block on
+    auto advance = [&](int which, int &r, int &kb) {   // move a cursor one K block on
         if (kb + 1 < QK) {
             kb += 1;
 #pragma unroll
             for (int d = 0; d < NDMA; d++)
-                if ((d >= TN) == first_group) dsrc[d] += dma_step(d);
-            if (first_group) sb_off1 += QN;
+                if ((d >= TN) == (which == 1)) dsrc[d] += dma_step(d);
         } else {
             r += 1;
             kb = 0;
-            seek(first_group, r, 0);
+            seek(which, r, 0);
         }
     };
 
@@ -211,24 +218,22 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
         // cold start: stage 0 <- block 0 of the first tile, then its first operands; stage 1 <- start of block 1
 #pragma unroll
         for (int d = 0; d < NDMA; d++) issue_dma(d, 0, dma_src(d, m0_cur, n0_cur, 0));
-        sb_cur = SB[nb_of(n0_cur) + vzero];
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        asm volatile("" : "+v"(sb_cur));
         __syncthreads();
         read_bfrag(0, 0);
         read_afrag(0, 0, 0);
         read_scales(0);
 #pragma unroll
         for (int i = 1; i < TN; i++) read_bfrag(i, 0);
-        // cursor 1 at block 1 (QK >= 2); its instructions d < TN ... belong to cursor 2, which starts at block 1 too
-        // for this one partial batch and then moves on to block 2
+        // cursor 2 issues its part of block 1 here and moves on to block 2 (or the next tile); cursor 1 stands at
+        // block 1 (QK >= 2)
         c2_r = 0; c2_kb = 1;
-        seek(false, 0, 1);
+        seek(2, 0, 1);
 #pragma unroll
         for (int d = 0; d < TN && d < NDMA; d++) issue_dma(d, 1, dsrc[d]);
-        advance(false, c2_r, c2_kb);                  // cursor 2 -> block 2 (or the next tile)
+        advance(2, c2_r, c2_kb);
         c1_r = 0; c1_kb = 1;
-        seek(true, 0, 1);
+        seek(1, 0, 1);
     }
 
     // one K block of the current tile; cur = the LDS stage it reads
@@ -236,18 +241,16 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
         constexpr int cur = decltype(cur_c)::value, nxt = 1 - cur;
         const float s_last = s[TM - 1];
 #pragma unroll
-        for (int j = 0; j < TM; j++) s[j] = sraw[j] * sb_cur;
+        for (int j = 0; j < TM; j++) s[j] = sraw[j] * sb_raw;
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int t = 0; t < NMFMA; t++) {
             const int j = t / TN, i = t % TN;
             if (t == BAR_SLOT) {
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                asm volatile("" : "+v"(sb_next));
+                wait_for_stage();
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (t == 0) sb_next = SB[sb_off1 + vzero];
             pring[t % PR] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
                 bfrag[i], afrag[j & 1], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
             asm volatile("" : "+v"(pring[t % PR]));
@@ -277,9 +280,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        sb_cur = sb_next;
-        advance(true, c1_r, c1_kb);
-        advance(false, c2_r, c2_kb);
+        advance(1, c1_r, c1_kb);
+        advance(2, c2_r, c2_kb);
     };
 
     for (int r = 0; r < my_tiles; r++) {

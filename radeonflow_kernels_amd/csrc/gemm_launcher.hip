@@ -57,11 +57,6 @@ struct Variant {
               rf::gemm_fp8_blockscale_streamk<BM, BN, WM, WN>,                             \
               rf::gemm_fp8_blockscale_persistent<BM, BN, WM, WN>,                          \
               rf::PersistentGeom<BM, BN, WM, WN>::LDS_BYTES }
-// the same kernel with NS LDS stages (deeper prefetch for shapes with few workgroups); no stream-K / persistent form
-#define RF_VARIANT_STAGES(BM, BN, WM, WN, NS)                                              \
-    Variant { BM, BN, WM, WN, rf::TileGeom<BM, BN, WM, WN, NS>::LDS_BYTES,                 \
-              rf::gemm_fp8_blockscale_tile<BM, BN, WM, WN, false, NS>,                     \
-              rf::gemm_fp8_blockscale_tile<BM, BN, WM, WN, true, NS>, nullptr, nullptr, 0 }
 // tiles with sides that are not powers of two (A fragments held, B streamed)
 #define RF_VARIANT_HOLD_A(BM, BN, WM, WN)                                                  \
     Variant { BM, BN, WM, WN, rf::HoldAGeom<BM, BN, WM, WN>::LDS_BYTES,                    \
@@ -74,10 +69,6 @@ const Variant kVariants[] = {
     RF_VARIANT(128, 256, 2, 4),   // 3: 8 waves, wave tile 64 x 64, 96 KiB LDS
     RF_VARIANT(128, 64, 2, 1),    // 4: 2 waves, wave tile 64 x 64, 48 KiB LDS (3 workgroups per CU)
     RF_VARIANT_HOLD_A(192, 288, 4, 2),   // 5: 8 waves, wave tile 48 x 144, 122 KiB LDS (6144 x 4608 = 512 tiles)
-    RF_VARIANT_STAGES(128, 256, 2, 4, 3),   // 6: as 3 with three stages, 146 KiB LDS
-    RF_VARIANT_STAGES(256, 128, 2, 2, 3),   // 7: as 2 with three stages, 147 KiB LDS
-    RF_VARIANT_STAGES(128, 128, 2, 2, 4),   // 8: as 1 with four stages, 131 KiB LDS
-    RF_VARIANT_STAGES(128, 64, 2, 1, 4),    // 9: as 4 with four stages, 99 KiB LDS
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
