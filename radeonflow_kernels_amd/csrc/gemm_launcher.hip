@@ -174,26 +174,39 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, rf_gemm_confi
             out->stream_k = p.stream_k;
             return;
         }
+    // No measured entry: a cost model fitted to the tuner's measurements of the tabled shapes (it lands within 10 % of
+    // the best measured plan on every one of them). Time in microseconds of a plan =
+    //   rounds * (K blocks per workgroup * c + f)           one workgroup per tile and K split
+    //   rounds * K blocks * c + f + (rounds - 1) * f_next   persistent: only the first tile starts cold
+    //   + reduction cost when K is split
+    // with rounds = ceil(workgroups / CUs). Only the 256x256 and 128x256 tiles are candidates: the smaller ones never
+    // won by more than a few percent.
+    struct Candidate { int variant; double c, f; };
+    const Candidate cands[] = {{0, 1.355, 9.46}, {3, 0.769, 3.61}};
+    const double f_next = 3.61, reduce_fixed = 6.83, reduce_per_elem = 8.7e-7;
+    const int splits_tried[] = {1, 2, 3, 4, 6, 8, 12, 16};
     const int qk = k / rf::BK;
-    int best = 1;
-    long tiles_big = (long)ceil_div(m, 256) * ceil_div(n, 256);
-    if (tiles_big >= num_cu) {
-        // stream_k stays off here: cutting tiles at arbitrary K blocks puts the workgroups of an XCD at different K
-        // positions, they stop sharing A/B lines in L2, and that costs more than the uneven last round (measured)
-        best = 0;
-    }
-    out->variant = best;
-    const Variant &v = kVariants[best];
-    // more tiles than CUs: let one pipeline run across the tiles of a workgroup when the shape allows it (measured
-    // gain 1 % at K = 7168, 3-7 % at K = 2048, 17 % at K = 256)
-    if (tiles_big > num_cu && persistent_ok(v, m, n, k)) out->stream_k = RF_SCHEDULE_PERSISTENT;
-    long tiles = (long)ceil_div(m, v.bm) * ceil_div(n, v.bn);
-    long slots = (long)num_cu * (best == 1 ? 2 : 1);
-    if (tiles < slots && qk >= 4) {
-        int s = (int)(slots / tiles);
-        if (s > 8) s = 8;
-        while (s > 1 && qk / s < 2) s--;
-        out->split_k = s < 1 ? 1 : s;
+    double best_cost = 1e30;
+    for (const Candidate &cd : cands) {
+        const Variant &v = kVariants[cd.variant];
+        const long tiles = (long)ceil_div(m, v.bm) * ceil_div(n, v.bn);
+        for (int sp : splits_tried) {
+            if (sp > qk) break;
+            const int kb_per = ceil_div(qk, sp), splits = ceil_div(qk, kb_per);
+            const long rounds = (tiles * splits + num_cu - 1) / num_cu;
+            for (int sched : {RF_SCHEDULE_TILES, RF_SCHEDULE_PERSISTENT}) {
+                if (sched == RF_SCHEDULE_PERSISTENT && (splits != 1 || !persistent_ok(v, m, n, k))) continue;
+                double t = sched == RF_SCHEDULE_PERSISTENT ? rounds * kb_per * cd.c + cd.f + (rounds - 1) * f_next
+                                                           : rounds * (kb_per * cd.c + cd.f);
+                if (splits > 1) t += reduce_fixed + reduce_per_elem * splits * (double)m * n;
+                if (t < best_cost) {
+                    best_cost = t;
+                    out->variant = cd.variant;
+                    out->split_k = sp;
+                    out->stream_k = sched;
+                }
+            }
+        }
     }
 }
 
