@@ -436,7 +436,7 @@ int launch_quantize(const void *x, int rows, int k, void *out, float *scales, hi
     }
     const bool vector_store = rows % 16 == 0 && (uintptr_t)out % 16 == 0;
     const int row_blocks = ceil_div(rows, 128);
-    dim3 grid(row_blocks, k / rf::BK);
+    dim3 grid(k / rf::BK, row_blocks);
     hipLaunchKernelGGL((rf::quantize_block128<PER_ROW, IN_BF16>), grid, dim3(256), 0, stream, x, rows, k, (uint8_t *)out,
                        scales, PER_ROW ? rows : row_blocks, vector_store);
     RF_HIP(hipGetLastError());

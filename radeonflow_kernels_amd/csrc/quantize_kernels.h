@@ -15,20 +15,21 @@
 namespace rf {
 
 // fp32 -> OCP e4m3fn code, round to nearest even, anything that rounds above 448 (and NaN) becomes NaN (0x7F).
-// Integer/exact-float arithmetic only, so that it agrees bit for bit with a CPU implementation.
+// Integer/exact-float arithmetic only, so that it agrees bit for bit with a CPU implementation; no branches.
 __device__ __forceinline__ uint32_t f32_to_e4m3fn_code(float f) {
     const uint32_t u = __builtin_bit_cast(uint32_t, f);
     const uint32_t sign = (u >> 24) & 0x80u, abits = u & 0x7fffffffu;
-    if (abits > 0x7f800000u) return sign | 0x7Fu;             // NaN
     const int e = (int)(abits >> 23) - 127;                   // floor(log2 |f|) for normal inputs
     int q = e - 3;                                            // exponent of the rounding quantum: 3 mantissa bits
-    if (q < -9) q = -9;                                       // subnormal range of e4m3: quantum 2^-9
+    q = q < -9 ? -9 : q;                                      // subnormal range of e4m3: quantum 2^-9
+    q = q > 120 ? 120 : q;                                    // Inf / NaN: keep the factor below finite
     const float inv_quantum = __builtin_bit_cast(float, (uint32_t)(127 - q) << 23);
     const float r = __builtin_rintf(__builtin_bit_cast(float, abits) * inv_quantum);   // exact product, RNE to integer
-    // r is in [0,16]; code = exponent field (q+10) and mantissa r-8, which also covers the subnormal codes (q = -9)
-    // and the carry r == 16 into the next exponent
-    const int code = ((q + 10) << 3) + (int)r - 8;
-    return sign | (uint32_t)(code > 126 ? 0x7F : code);
+    // r is in [0,16] for finite inputs; code = exponent field (q+10) and mantissa r-8, which also covers the subnormal
+    // codes (q = -9) and the carry r == 16 into the next exponent
+    const bool finite = abits < 0x7f800000u;
+    const int code = ((q + 10) << 3) + (int)(finite ? r : 0.f) - 8;
+    return sign | (uint32_t)((code > 126 || !finite) ? 0x7F : code);
 }
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __builtin_bit_cast(float, h << 16); }
@@ -47,7 +48,9 @@ __global__ __launch_bounds__(256) void quantize_block128(const void *__restrict_
     auto row_of = [&](int i) { return 32 * (i >> 2) + 4 * (int)(threadIdx.x >> 5) + (i & 3); };
     __shared__ float wave_max[4];
     const int t = threadIdx.x, lane32 = t & 31;
-    const int r0 = blockIdx.x * 128, kb = blockIdx.y, k0 = kb * 128;
+    // K blocks vary fastest over the grid: workgroups that run together read neighbouring 512-byte (256-byte) pieces
+    // of the same source rows
+    const int rb = blockIdx.y, r0 = rb * 128, kb = blockIdx.x, k0 = kb * 128;
     float v[16][4];
 #pragma unroll
     for (int i = 0; i < 16; i++) {
@@ -97,9 +100,11 @@ __global__ __launch_bounds__(256) void quantize_block128(const void *__restrict_
         const float sb = a > 0.f ? a / 448.0f : 1.0f;
 #pragma unroll
         for (int i = 0; i < 16; i++) s[i] = sb;
-        if (t == 0) scales[(size_t)kb * scale_ld + blockIdx.x] = sb;
+        if (t == 0) scales[(size_t)kb * scale_ld + rb] = sb;
     }
-    // quantise and transpose through LDS: tile[k][row]
+    // quantise and transpose through LDS: tile[k][row]. (Replacing the 64 divisions per thread by a multiplication
+    // with 1/scale plus an exact fallback near rounding boundaries was tried and is bit-exact, but no faster: the
+    // kernel is bound by its memory access pattern, not by the ALU.)
 #pragma unroll
     for (int i4 = 0; i4 < 4; i4++)
 #pragma unroll

@@ -26,6 +26,19 @@ def _source(rows, k, seed, kind):
         x[: min(rows, 3), :128] = 0.0
         x[rows // 2, k // 2] = 3.0e38
         x[rows - 1, k - 1] = 1.0e-41        # fp32 denormal
+    if kind == "boundary":      # quotients x/scale within a few fp32 ulps of the midpoints between fp8 codes
+        rng = np.random.default_rng(seed)
+        amax = np.exp2(rng.integers(-20, 20, (rows, k // 128, 1))).astype(np.float32) * rng.uniform(1, 2, (rows, k // 128, 1)).astype(np.float32)
+        codes = np.arange(0, 126, dtype=np.uint8)
+        vals = cref.e4m3fn_to_f32(codes)
+        mids = ((vals[:-1] + vals[1:]) / 2).astype(np.float32)                   # exact in fp32
+        pick = mids[rng.integers(0, len(mids), (rows, k // 128, 128))]
+        scale = (amax / np.float32(448.0)).astype(np.float32)
+        x = (pick * scale).astype(np.float32)
+        x = (x.view(np.int32) + rng.integers(-3, 4, x.shape).astype(np.int32)).view(np.float32)   # +-3 ulp
+        x *= rng.choice(np.array([-1.0, 1.0], np.float32), x.shape)
+        x[:, :, 0] = amax[:, :, 0]                                             # pin the block maximum
+        x = x.reshape(rows, k)
     return np.ascontiguousarray(x, dtype=np.float32)
 
 
@@ -34,7 +47,7 @@ def _unpack(q, s):
     return q.T.contiguous().view(torch.uint8).cpu().numpy(), s.T.contiguous().cpu().numpy()
 
 
-@pytest.mark.parametrize("kind", ["normal", "wide"])
+@pytest.mark.parametrize("kind", ["normal", "wide", "boundary"])
 @pytest.mark.parametrize("rows,k", [(128, 128), (256, 512), (1024, 7168), (576, 1024), (200, 256), (1, 128), (33, 384),
                                     (6144, 256)])
 def test_quantize_a_matches_oracle_bit_for_bit(rfk, rows, k, kind):
@@ -48,7 +61,7 @@ def test_quantize_a_matches_oracle_bit_for_bit(rfk, rows, k, kind):
     assert np.array_equal(a_gpu, np.asarray(a_ref))
 
 
-@pytest.mark.parametrize("kind", ["normal", "wide"])
+@pytest.mark.parametrize("kind", ["normal", "wide", "boundary"])
 @pytest.mark.parametrize("rows,k", [(128, 128), (256, 512), (1536, 7168), (576, 1024), (200, 256), (1, 128), (33, 384)])
 def test_quantize_b_matches_oracle_bit_for_bit(rfk, rows, k, kind):
     w = _source(rows, k, 2000 + rows + k, kind)
