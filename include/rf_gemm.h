@@ -117,11 +117,15 @@ int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const flo
  *                    writes a ([K][M] fp8, the layout `run` takes) and as ([K/128][M] fp32).
  *   rf_quantize_b_*: w is [n][k] row-major, one scale per 128x128 block (the last N block may be partial);
  *                    writes b ([K][N] fp8) and bs ([K/128][ceil(N/128)] fp32).
- * k must be a positive multiple of 128; sources 16-byte aligned (bf16: 8). Enqueued on `stream`. */
+ * k must be a positive multiple of 128; sources 16-byte aligned. Enqueued on `stream`. */
 int rf_quantize_a_f32(const float *x, int m, int k, void *a, float *as, hipStream_t stream);
 int rf_quantize_a_bf16(const void *x, int m, int k, void *a, float *as, hipStream_t stream);
 int rf_quantize_b_f32(const float *w, int n, int k, void *b, float *bs, hipStream_t stream);
 int rf_quantize_b_bf16(const void *w, int n, int k, void *b, float *bs, hipStream_t stream);
+
+/* Elementwise cast fp32 -> OCP e4m3fn (round to nearest even; |x| that rounds above 448, infinities and NaN become
+ * NaN with the sign kept), the conversion the quantisers apply after scaling. No counterpart in the reference. */
+int rf_cast_f32_to_e4m3fn(const float *x, size_t count, void *out, hipStream_t stream);
 
 /* Text of the last failure on this thread's most recent rf_* call ("" if none). */
 const char *rf_gemm_last_error(void);

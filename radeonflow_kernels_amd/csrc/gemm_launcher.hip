@@ -426,8 +426,8 @@ int launch_quantize(const void *x, int rows, int k, void *out, float *scales, hi
         return fail(RF_ERR_BAD_SHAPE, "unsupported shape rows=" + std::to_string(rows) + " K=" + std::to_string(k) +
                                           " (need rows>=1, K a positive multiple of 128)");
     if (!x || !out || !scales) return fail(RF_ERR_NULL_POINTER, "null device pointer");
-    if ((uintptr_t)x % (IN_BF16 ? 8 : 16) != 0 || (uintptr_t)scales % 4 != 0)
-        return fail(RF_ERR_BAD_CONFIG, "source must be 16-byte aligned (8 for bf16), scales 4-byte aligned");
+    if ((uintptr_t)x % 16 != 0 || (uintptr_t)scales % 4 != 0)
+        return fail(RF_ERR_BAD_CONFIG, "source must be 16-byte aligned, scales 4-byte aligned");
     State &s = state();
     {
         std::lock_guard<std::mutex> lock(s.mu);
@@ -530,6 +530,18 @@ int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const flo
     }
     hipLaunchKernelGGL(v.kernel, dim3(tiles), dim3(v.threads), v.lds, stream, (const uint8_t *)a, (const uint8_t *)b, as,
                        bs, (uint16_t *)c, m_total, n, k, groups, tiles_n, 8, table);
+    RF_HIP(hipGetLastError());
+    return RF_OK;
+}
+
+int rf_cast_f32_to_e4m3fn(const float *x, size_t count, void *out, hipStream_t stream) {
+    g_last_error.clear();
+    if (count == 0) return RF_OK;
+    if (!x || !out) return fail(RF_ERR_NULL_POINTER, "null device pointer");
+    if ((uintptr_t)x % 16 != 0 || (uintptr_t)out % 4 != 0)
+        return fail(RF_ERR_BAD_CONFIG, "source must be 16-byte aligned, destination 4-byte aligned");
+    hipLaunchKernelGGL(rf::cast_f32_to_e4m3fn, dim3((unsigned)((count + 1023) / 1024)), dim3(256), 0, stream, x,
+                       (uint8_t *)out, count);
     RF_HIP(hipGetLastError());
     return RF_OK;
 }

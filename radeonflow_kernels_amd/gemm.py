@@ -39,7 +39,8 @@ class PerfMetrics(ctypes.Structure):
 
 EXPORTS = ("run", "rf_fp8_gemm", "rf_fp8_gemm_ex", "rf_gemm_select_config", "rf_gemm_num_variants",
            "rf_gemm_variant_info", "rf_gemm_variant_has_stream_k", "rf_gemm_variant_has_persistent", "rf_gemm_workspace_bytes", "rf_gemm_init", "rf_gemm_destroy",
-           "rf_gemm_last_error", "rf_fp8_gemm_grouped", "rf_quantize_a_f32", "rf_quantize_a_bf16", "rf_quantize_b_f32", "rf_quantize_b_bf16")
+           "rf_gemm_last_error", "rf_fp8_gemm_grouped", "rf_quantize_a_f32", "rf_quantize_a_bf16", "rf_quantize_b_f32", "rf_quantize_b_bf16",
+           "rf_cast_f32_to_e4m3fn")
 
 
 def lib():
@@ -78,6 +79,8 @@ def lib():
             f = getattr(L, name)
             f.argtypes = [ctypes.c_void_p, i32, i32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
             f.restype = i32
+        L.rf_cast_f32_to_e4m3fn.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_void_p]
+        L.rf_cast_f32_to_e4m3fn.restype = i32
         _lib = L
     return _lib
 
@@ -182,6 +185,19 @@ def _quantize(x, per_row):
     if rc != RF_OK:
         raise RuntimeError("%s failed (%d): %s" % (name, rc, last_error()))
     return q.T, scales.T         # the transposed views fp8_mm takes: [rows, K] stride (1, rows), [rows or QN, K/128]
+
+
+def cast_to_e4m3fn(x):
+    """fp32 tensor (contiguous, on the GPU) -> torch.float8_e4m3fn tensor of the same shape, round to nearest even."""
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise ValueError("source must be a contiguous fp32 tensor")
+    out = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device=x.device)
+    stream = ctypes.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)
+    with torch.cuda.device(x.device):
+        rc = lib().rf_cast_f32_to_e4m3fn(x.data_ptr(), x.numel(), out.data_ptr(), stream)
+    if rc != RF_OK:
+        raise RuntimeError("rf_cast_f32_to_e4m3fn failed (%d): %s" % (rc, last_error()))
+    return out
 
 
 def quantize_a(x):

@@ -109,6 +109,25 @@ def test_quantise_then_gemm_end_to_end(rfk):
     assert_close_to_oracle(out, exp, RTOL, ATOL, "quantise + gemm")
 
 
+def test_cast_matches_the_oracle_encoder_on_a_dense_sweep_of_all_floats(rfk):
+    """Every 61st fp32 bit pattern (70 million values: all binades, denormals, infinities, NaNs of both signs) and a
+    dense neighbourhood of every boundary between fp8 codes."""
+    bits = np.arange(0, 2 ** 32, 61, dtype=np.uint64).astype(np.uint32)
+    vals = cref.e4m3fn_to_f32(np.arange(0, 127, dtype=np.uint8))
+    mids = np.concatenate([(vals[:-1] + vals[1:]) / 2, [464.0, 448.0, 480.0]]).astype(np.float32)
+    near = (mids.view(np.uint32)[:, None].astype(np.int64) + np.arange(-40, 41)[None, :]).astype(np.uint32).ravel()
+    bits = np.concatenate([bits, near, near | np.uint32(0x80000000)])
+    bits = bits[: bits.size // 4 * 4 + 0]
+    x = torch.from_numpy(bits.view(np.float32).copy())
+    got = rfk.cast_to_e4m3fn(x.cuda()).view(torch.uint8).cpu().numpy()
+    exp = cref.f32_to_e4m3fn(x.numpy())
+    bad = np.nonzero(got != exp)[0]
+    assert bad.size == 0, "first mismatch: bits %08x got %02x expected %02x" % (bits[bad[0]], got[bad[0]], exp[bad[0]])
+    # a tail that is not a multiple of four
+    y = torch.from_numpy(bits[:1027].view(np.float32).copy()).cuda()
+    assert np.array_equal(rfk.cast_to_e4m3fn(y).view(torch.uint8).cpu().numpy(), exp[:1027])
+
+
 def test_status_codes(rfk):
     L = rfk.lib()
     x = torch.zeros((128, 128), device="cuda")
