@@ -499,6 +499,37 @@ __device__ __forceinline__ void store_tile_f32(const f32x4 (&acc)[BM / WAVES_M /
     }
 }
 
+// The same through LDS, one m-tile (16 rows) of every wave per pass, written out 16 bytes per lane with neighbouring
+// lanes along a row: each store instruction covers whole rows of the wave tile (256 contiguous bytes for 64 columns)
+// instead of sixteen 64-byte pieces. Starts with a barrier like store_tile_bf16 (the regions overlay the stages).
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+__device__ __forceinline__ void store_tile_f32_staged(const f32x4 (&acc)[BM / WAVES_M / 16][BN / WAVES_N / 16],
+                                                      float *__restrict__ t, size_t ld, int m_lim, int n_lim,
+                                                      uint8_t *staging) {
+    using G = TileGeom<BM, BN, WAVES_M, WAVES_N>;
+    constexpr int ROW = G::WN * 4 + 16, REGION = 16 * ROW;
+    constexpr int LPR = G::WN / 4, RPI = 64 / LPR;        // lanes per row (16 bytes each), rows per store instruction
+    static_assert(G::NW * REGION <= 2 * G::STAGE && 64 % LPR == 0 && 16 % RPI == 0, "staging geometry");
+    int vz;                                  // see store_tile_bf16
+    asm volatile("v_mov_b32 %0, 0" : "=v"(vz));
+    const int lane = (threadIdx.x & 63) + vz, wave = threadIdx.x >> 6, L = lane & 15, g = lane >> 4;
+    const int wm = wave % WAVES_M, wn = wave / WAVES_M;
+    uint8_t *region = staging + wave * REGION;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < G::TM; j++) {
+#pragma unroll
+        for (int i = 0; i < G::TN; i++) *(f32x4 *)(region + L * ROW + (16 * i + 4 * g) * 4) = acc[j][i];
+#pragma unroll
+        for (int r0 = 0; r0 < 16; r0 += RPI) {
+            const int r = r0 + lane / LPR, cb = (lane % LPR) * 16;
+            const uint4 v = *(const uint4 *)(region + r * ROW + cb);
+            const int m = wm * G::WM + 16 * j + r, n = wn * G::WN + cb / 4;
+            if (m < m_lim && n < n_lim) *(uint4 *)(t + (size_t)m * ld + n) = v;
+        }
+    }
+}
+
 // Partial tiles exchanged between workgroups of the stream-K grid. The two workgroups may sit on different XCDs,
 // whose L2 caches are not coherent with each other. Instead of device-wide fences (which write back and invalidate
 // a whole L2, throwing away the A/B tiles every other workgroup on the XCD is re-using), each access carries system
@@ -551,8 +582,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
     f32x4 acc[G::TM][G::TN];
     tile_mainloop<BM, BN, WAVES_M, WAVES_N, NS>(A, B, SA, SB, M, M, N, m0, n0, kb_begin, kb_end, lds, acc);
     if constexpr (PARTIAL)
-        store_tile_f32<BM, BN, WAVES_M, WAVES_N>(acc, (float *)Cout + ((size_t)blockIdx.y * M + m0) * N + n0, N, M - m0,
-                                                 N - n0);
+        store_tile_f32_staged<BM, BN, WAVES_M, WAVES_N>(acc, (float *)Cout + ((size_t)blockIdx.y * M + m0) * N + n0, N,
+                                                        M - m0, N - n0, lds);
     else
         store_tile_bf16<BM, BN, WAVES_M, WAVES_N>(acc, (uint16_t *)Cout, M, N, m0, n0, lds);
 }
