@@ -278,6 +278,19 @@ def main():
                           "us": round(u, 2), "tflops": round(tf, 1), "pct_fp8_mfma_peak": round(100 * tf / PEAK_FP8_TFLOPS, 2)}
         print("grouped %s: %.2f us  %.1f TFLOP/s (%.1f %% of peak)" % (out["grouped"]["workload"], u, tf,
               100 * tf / PEAK_FP8_TFLOPS), file=sys.stderr)
+        # what the chip sustains on the same MFMA instruction from registers alone (clock under its power limit);
+        # run as a child process once the GEMM work above is done
+        probe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "radeonflow_kernels_amd", "lib", "mfma_ceiling")
+        if os.path.exists(probe):
+            import subprocess
+            torch.cuda.synchronize()
+            r = subprocess.run([probe, "0.3"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=60)
+            if r.returncode == 0:
+                out["mfma_ceiling"] = json.loads(r.stdout.strip().splitlines()[-1])
+                out["mfma_ceiling"]["gemm_pct_of_normal_ceiling"] = round(100 * out["value"] / out["mfma_ceiling"]["normal"], 2)
+                print("register-only MFMA ceiling: %r" % (out["mfma_ceiling"],), file=sys.stderr)
+            else:
+                print("mfma_ceiling failed: %s" % r.stderr.strip(), file=sys.stderr)
     print(json.dumps(out))
     return 0
 

@@ -63,8 +63,19 @@ def build_checker(verbose=False):
     return out
 
 
+def build_probe(verbose=False):
+    """lib/mfma_ceiling: register-only MFMA throughput of the whole chip (bench.py --all reports it beside the GEMM)."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    out = os.path.join(LIB_DIR, "mfma_ceiling")
+    res = _run([hipcc()] + HIPCC_FLAGS + ["-o", out, os.path.join(CSRC, "mfma_ceiling.hip")])
+    if verbose and res:
+        print(res)
+    return out
+
+
 def build_all(verbose=False):
     build_lib(verbose)
+    build_probe(verbose)
     build_checker(verbose)
 
 

@@ -138,10 +138,19 @@ __device__ __forceinline__ void tile_mainloop(
     constexpr int NSC = BM / 64;                                                // scale loads: 64 floats each
     static_assert(STAGE_A % (1024 * NW) == 0 && STAGE_B % (1024 * NW) == 0, "loads must divide evenly over waves");
     static_assert(NSC <= NW, "one scale load per wave at most");
-    static_assert(WN <= 128 && 128 % WN == 0, "a wave's N range must sit inside one scale block");
-    static_assert(TM % 4 == 0, "scales are read back four at a time");
+    // ONE_SB: the wave's columns lie inside one 128-column b_scale block. Otherwise (tile sides that are not powers
+    // of two) they may straddle two: n-tiles below a wave-uniform split use the first block's scale, the others the
+    // second's, and the K loop is instantiated once per possible split.
+    constexpr bool ONE_SB = WN <= 128 && 128 % WN == 0;
+    static_assert(ONE_SB || (TN == 3 && WN < 128), "straddling waves: three n-tiles, split before n-tile 1 or 2");
+    static_assert(TM % 2 == 0, "scales are read back two or four at a time");
     constexpr int CPR_A = BM / 16, CPR_B = BN / 16;          // 16-byte chunks per LDS row
-    constexpr int RPI_A = 1024 / BM, RPI_B = 1024 / BN;      // rows per load instruction
+    // EVEN: a 1 KiB load instruction covers whole rows (RPI of them). Otherwise instruction q covers the 64 chunks
+    // from linear chunk 64q of the stage, a wave's instructions together cover whole rows (ROWS_W of them).
+    constexpr bool EVEN_A = 1024 % BM == 0, EVEN_B = 1024 % BN == 0;
+    constexpr int RPI_A = EVEN_A ? 1024 / BM : 0, RPI_B = EVEN_B ? 1024 / BN : 0;      // rows per load instruction
+    constexpr int ROWS_W_A = INST_A * 64 / CPR_A, ROWS_W_B = INST_B * 64 / CPR_B;      // rows per wave
+    static_assert((INST_A * 64) % CPR_A == 0 && (INST_B * 64) % CPR_B == 0, "a wave's loads cover whole rows");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -155,33 +164,45 @@ __device__ __forceinline__ void tile_mainloop(
     // Load instruction i of this wave covers rows (wave*INST + i)*RPI .. +RPI-1. Its per-lane offset differs from
     // that of another instruction only by a wave-uniform amount when both see the same row swizzle, i.e. the same
     // (k & 7) and (k >> 5) & 1 for every lane. So only one VGPR per swizzle class is kept; the rest is scalar.
-    constexpr int PER_A = (8 / RPI_A) > 0 ? (8 / RPI_A) : 1, PER_B = (8 / RPI_B) > 0 ? (8 / RPI_B) : 1;
+    // (Rows that are not a power of two wide: every instruction of a wave keeps its own offset register.)
+    constexpr int PER_A = !EVEN_A ? 1 : (8 / RPI_A) > 0 ? (8 / RPI_A) : 1, PER_B = !EVEN_B ? 1 : (8 / RPI_B) > 0 ? (8 / RPI_B) : 1;
     constexpr int GRP_A = (INST_A * RPI_A + 31) / 32, GRP_B = (INST_B * RPI_B + 31) / 32;   // 32-row groups per wave
-    constexpr int NCLS_A = (PER_A < INST_A ? PER_A : INST_A) * GRP_A, NCLS_B = (PER_B < INST_B ? PER_B : INST_B) * GRP_B;
-    static_assert((INST_A * RPI_A) % 32 == 0 || INST_A * RPI_A < 32, "a wave's rows cover whole 32-row groups");
-    static_assert((INST_B * RPI_B) % 32 == 0 || INST_B * RPI_B < 32, "a wave's rows cover whole 32-row groups");
-    auto cls_a = [](int i) { return i % PER_A + PER_A * (i * RPI_A / 32); };   // class of instruction i
-    auto rep_a = [](int c) { return c % PER_A + (c / PER_A) * (32 / RPI_A); }; // first instruction of class c
-    auto cls_b = [](int i) { return i % PER_B + PER_B * (i * RPI_B / 32); };
-    auto rep_b = [](int c) { return c % PER_B + (c / PER_B) * (32 / RPI_B); };
+    constexpr int NCLS_A = !EVEN_A ? INST_A : (PER_A < INST_A ? PER_A : INST_A) * GRP_A;
+    constexpr int NCLS_B = !EVEN_B ? INST_B : (PER_B < INST_B ? PER_B : INST_B) * GRP_B;
+    static_assert(!EVEN_A || (INST_A * RPI_A) % 32 == 0 || INST_A * RPI_A < 32, "a wave's rows cover whole 32-row groups");
+    static_assert(!EVEN_B || (INST_B * RPI_B) % 32 == 0 || INST_B * RPI_B < 32, "a wave's rows cover whole 32-row groups");
+    auto cls_a = [](int i) { return !EVEN_A ? i : i % PER_A + PER_A * (i * RPI_A / 32); };   // class of instruction i
+    auto rep_a = [](int c) { return !EVEN_A ? c : c % PER_A + (c / PER_A) * (32 / (EVEN_A ? RPI_A : 1)); };   // first instruction of class c
+    auto cls_b = [](int i) { return !EVEN_B ? i : i % PER_B + PER_B * (i * RPI_B / 32); };
+    auto rep_b = [](int c) { return !EVEN_B ? c : c % PER_B + (c / PER_B) * (32 / (EVEN_B ? RPI_B : 1)); };
     uint32_t goff_a[NCLS_A], goff_b[NCLS_B], goff_s, goff_sb;
 #pragma unroll
     for (int c_ = 0; c_ < NCLS_A; c_++) {
-        int q = wave * INST_A + rep_a(c_);
-        int kl = q * RPI_A + lane / CPR_A;
-        int c = (lane % CPR_A) ^ swizzle_of_row<BM>(kl);
+        int rl, ch, kl;                                       // row relative to the instruction's scalar base, chunk, stage row
+        if constexpr (EVEN_A) {
+            rl = lane / CPR_A, ch = lane % CPR_A, kl = (wave * INST_A + rep_a(c_)) * RPI_A + rl;
+        } else {
+            const int ql = rep_a(c_) * 64 + lane;
+            rl = ql / CPR_A, ch = ql % CPR_A, kl = wave * ROWS_W_A + rl;
+        }
+        int c = ch ^ swizzle_of_row<BM>(kl);
         int m = m0 + c * 16;
         if (m + 16 > M) m = M - 16;                           // rows past M: any valid bytes will do
-        goff_a[c_] = (uint32_t)(lane / CPR_A) * (uint32_t)ldm + (uint32_t)m;
+        goff_a[c_] = (uint32_t)rl * (uint32_t)ldm + (uint32_t)m;
     }
 #pragma unroll
     for (int c_ = 0; c_ < NCLS_B; c_++) {
-        int q = wave * INST_B + rep_b(c_);
-        int kl = q * RPI_B + lane / CPR_B;
-        int c = (lane % CPR_B) ^ swizzle_of_row<BN>(kl);
+        int rl, ch, kl;
+        if constexpr (EVEN_B) {
+            rl = lane / CPR_B, ch = lane % CPR_B, kl = (wave * INST_B + rep_b(c_)) * RPI_B + rl;
+        } else {
+            const int ql = rep_b(c_) * 64 + lane;
+            rl = ql / CPR_B, ch = ql % CPR_B, kl = wave * ROWS_W_B + rl;
+        }
+        int c = ch ^ swizzle_of_row<BN>(kl);
         int n = n0 + c * 16;
         if (n + 16 > N) n = N - 16;
-        goff_b[c_] = (uint32_t)(lane / CPR_B) * (uint32_t)N + (uint32_t)n;
+        goff_b[c_] = (uint32_t)rl * (uint32_t)N + (uint32_t)n;
     }
     {
         // a_scale slot s of the stage holds the scale of row (s/WM)*WM + 16*(s%TM) + (s%WM)/TM of the tile, so that
@@ -212,8 +233,9 @@ __device__ __forceinline__ void tile_mainloop(
     const uint32_t lds_dst_a = lds_base + wave * (INST_A * 1024), lds_dst_b = lds_base + OFF_B + wave * (INST_B * 1024),
                    lds_dst_s = lds_base + OFF_S + wave * 256, lds_dst_sb = lds_base + OFF_S + OFF_SB;
     auto dma_src = [&](int d, int kb) -> const uint8_t * {
-        if (d < INST_A) return A + ((size_t)kb * BK + (size_t)(wave * INST_A + d) * RPI_A) * ldm;
-        if (d < D_SA) return B + ((size_t)kb * BK + (size_t)(wave * INST_B + (d - INST_A)) * RPI_B) * N;
+        if (d < INST_A) return A + ((size_t)kb * BK + (size_t)(EVEN_A ? (wave * INST_A + d) * RPI_A : wave * ROWS_W_A)) * ldm;
+        if (d < D_SA)
+            return B + ((size_t)kb * BK + (size_t)(EVEN_B ? (wave * INST_B + (d - INST_A)) * RPI_B : wave * ROWS_W_B)) * N;
         if (d == D_SA) return (const uint8_t *)(SA + (size_t)kb * ldm);
         return (const uint8_t *)(SB + (size_t)kb * QN);
     };
@@ -247,15 +269,30 @@ __device__ __forceinline__ void tile_mainloop(
     // ---- LDS -> MFMA operands: per-lane byte offsets of the transpose reads (stage 0, t = 0) ----
     // lane (L,g) of read t points at row k = 32g + 8t + L/2, half (L&1) of 16-byte chunk c.
     const int krow = 32 * g + (L >> 1);
-    // chunk index of m-tile j is (wm*TM + j) ^ sw = ((wm*TM) ^ sw) ^ j because j < TM and wm*TM is a multiple of TM
-    // (TM, TN powers of two): one base register per operand, the tile index is XORed in at the use.
-    static_assert((TM & (TM - 1)) == 0 && (TN & (TN - 1)) == 0, "tile counts are powers of two");
+    // chunk index of m-tile j is (wm*TM + j) ^ sw = ((wm*TM) ^ sw) ^ j when j < TM and wm*TM is a multiple of TM
+    // (TM, TN powers of two): one base register per operand, the tile index is XORed in at the use. Other tile counts
+    // keep one offset register per tile.
+    constexpr bool POW2_T = (TM & (TM - 1)) == 0 && (TN & (TN - 1)) == 0;
     const uint32_t aoff_base = krow * BM + (((wm * TM) ^ swizzle_of_row<BM>(krow)) << 4) + 8 * (L & 1);
     // (OFF_B has no low bits set, so it passes through the XOR with the tile index unchanged)
     const uint32_t boff_base = OFF_B + krow * BN + (((wn * TN) ^ swizzle_of_row<BN>(krow)) << 4) + 8 * (L & 1);
+    uint32_t aoff_tile[POW2_T ? 1 : TM], boff_tile[POW2_T ? 1 : TN];
+    if constexpr (!POW2_T) {
+#pragma unroll
+        for (int j = 0; j < TM; j++)
+            aoff_tile[j] = krow * BM + (((wm * TM + j) ^ swizzle_of_row<BM>(krow)) << 4) + 8 * (L & 1);
+#pragma unroll
+        for (int i = 0; i < TN; i++)
+            boff_tile[i] = OFF_B + krow * BN + (((wn * TN + i) ^ swizzle_of_row<BN>(krow)) << 4) + 8 * (L & 1);
+    }
     const uint32_t soff = OFF_S + (wm * WM + L * TM) * 4;               // this lane's TM scales
-    // this wave's b_scale: its columns lie in one 128-column block, the (nb - first block of the tile)-th slot
-    const uint32_t sboff = OFF_S + OFF_SB + ((((n0 + wn * WN) >> 7) - (n0 >> 7)) << 2);
+    // this wave's b_scale slots (slot = 128-column block - first block of the tile): n-tiles i < sb_split lie in the
+    // block of slot 0, the others in the next one
+    const int ncol0 = n0 + wn * WN;
+    const int sb_split_raw = (((ncol0 >> 7) + 1) * 128 - ncol0) >> 4;
+    const int sb_split = __builtin_amdgcn_readfirstlane(sb_split_raw < TN ? sb_split_raw : TN);
+    const uint32_t sboff = OFF_S + OFF_SB + (((ncol0 >> 7) - (n0 >> 7)) << 2);
+    const uint32_t sboff1 = sboff + (sb_split < TN ? 4 : 0);
 
 #pragma unroll
     for (int j = 0; j < TM; j++)
@@ -275,7 +312,8 @@ __device__ __forceinline__ void tile_mainloop(
     //     per slot, and run on into the first slots of the next iteration.
     // An empty volatile asm after each MFMA / fold anchors it in its slot, sched_barrier(0) keeps the slots apart;
     // the compiler still places the LDS waits and hazard nops.
-    constexpr int PR = 4, LAG = 3, NMFMA = TM * TN, BAR_SLOT = (TM - 1) * TN;
+    constexpr int NMFMA = TM * TN, PR = NMFMA % 4 == 0 ? 4 : 3, LAG = PR - 1, BAR_SLOT = (TM - 1) * TN;
+    static_assert(NMFMA % PR == 0, "ring positions repeat per K block");
     static_assert(LAG < TN && LAG < PR, "lagged folds of a K block stay inside its last m-tile row");
     static_assert(TM % 2 == 0, "the last m-tile uses afrag[1], so afrag[0] is free for the next block");
     static_assert(NDMA - TN <= BAR_SLOT, "the DMA batch finishes well before the barrier that needs it");
@@ -284,11 +322,13 @@ __device__ __forceinline__ void tile_mainloop(
 
     i32x8 bfrag[TN], afrag[2];
     f32x4 pring[PR];
-    float s[TM], sraw[TM], sb_raw = 0.f;
+    float s[TM], s1[ONE_SB ? 1 : TM], sraw[TM], sb_raw = 0.f, sb_raw1 = 0.f;   // s1: scales of the second b_scale block
 #pragma unroll
     for (int r = 0; r < PR; r++) pring[r] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int j = 0; j < TM; j++) s[j] = 0.f;
+#pragma unroll
+    for (int j = 0; j < (ONE_SB ? 1 : TM); j++) s1[j] = 0.f;
 
     auto rd = [&](uint32_t stage_base, uint32_t off) {
         return __builtin_amdgcn_ds_read_tr8_b64_v2i32((RF_LDS i32x2 *)(lds + stage_base + off));
@@ -296,7 +336,7 @@ __device__ __forceinline__ void tile_mainloop(
     auto read_bfrag = [&](int i, int stage) {
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-            i32x2 v = rd(stage * STAGE_B, (boff_base ^ (i << 4)) + t * 8 * BN);
+            i32x2 v = rd(stage * STAGE_B, (POW2_T ? boff_base ^ (i << 4) : boff_tile[POW2_T ? 0 : i]) + t * 8 * BN);
             bfrag[i][2 * t] = v[0];
             bfrag[i][2 * t + 1] = v[1];
         }
@@ -304,19 +344,29 @@ __device__ __forceinline__ void tile_mainloop(
     auto read_afrag = [&](int buf, int j, int stage) {
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-            i32x2 v = rd(stage * STAGE_A, (aoff_base ^ (j << 4)) + t * 8 * BM);
+            i32x2 v = rd(stage * STAGE_A, (POW2_T ? aoff_base ^ (j << 4) : aoff_tile[POW2_T ? 0 : j]) + t * 8 * BM);
             afrag[buf][2 * t] = v[0];
             afrag[buf][2 * t + 1] = v[1];
         }
     };
     auto read_scales = [&](int stage) {
+        if constexpr (TM % 4 == 0) {
 #pragma unroll
-        for (int q = 0; q < TM / 4; q++) {
-            f32x4 v = *(RF_LDS f32x4 *)(lds + stage * STAGE_S + soff + q * 16);
+            for (int q = 0; q < TM / 4; q++) {
+                f32x4 v = *(RF_LDS f32x4 *)(lds + stage * STAGE_S + soff + q * 16);
 #pragma unroll
-            for (int e = 0; e < 4; e++) sraw[4 * q + e] = v[e];
+                for (int e = 0; e < 4; e++) sraw[4 * q + e] = v[e];
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < TM / 2; q++) {
+                f32x2 v = *(RF_LDS f32x2 *)(lds + stage * STAGE_S + soff + q * 8);
+                sraw[2 * q] = v[0];
+                sraw[2 * q + 1] = v[1];
+            }
         }
         sb_raw = *(RF_LDS float *)(lds + stage * STAGE_S + sboff);
+        if constexpr (!ONE_SB) sb_raw1 = *(RF_LDS float *)(lds + stage * STAGE_S + sboff1);
     };
 
     if (kb_begin < kb_end) {
@@ -341,12 +391,18 @@ __device__ __forceinline__ void tile_mainloop(
 #pragma unroll
     for (int d = 0; d < NDMA; d++) dsrc[d] = dma_src(d, clamp_kb(kb_begin + (d < TN ? NS : NS - 1)));
     // one K block; cur is the stage it reads (compile-time: the loop below is unrolled NS times)
-    auto k_block = [&](auto cur_c, int kb) {
+    // split (compile-time): n-tiles i < split fold with s, the others with s1
+    auto k_block = [&](auto cur_c, auto split_c, int kb) {
         constexpr int cur = decltype(cur_c)::value, nxt = (cur + 1) % NS, prv = (cur + NS - 1) % NS;
+        constexpr int split = decltype(split_c)::value;
         const bool adv1 = kb + NS <= kb_last, adv2 = kb + NS + 1 <= kb_last;   // does the next iteration move on a block?
-        const float s_last = s[TM - 1];                    // scale of the previous block's last m-tile (lagged folds)
+        // scales of the previous block's last m-tile (lagged folds)
+        const float s_last = s[TM - 1], s1_last = s1[ONE_SB ? 0 : TM - 1];
 #pragma unroll
         for (int j = 0; j < TM; j++) s[j] = sraw[j] * sb_raw;
+        if constexpr (!ONE_SB)
+#pragma unroll
+            for (int j = 0; j < TM; j++) s1[j] = sraw[j] * sb_raw1;
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int t = 0; t < NMFMA; t++) {
@@ -386,35 +442,42 @@ __device__ __forceinline__ void tile_mainloop(
             if (t >= LAG) {
                 const int u = t - LAG, ju = u / TN, iu = u % TN;
 #pragma unroll
-                for (int e = 0; e < 4; e++) acc[ju][iu][e] = __builtin_fmaf(s[ju], pring[u % PR][e], acc[ju][iu][e]);
+                for (int e = 0; e < 4; e++)
+                    acc[ju][iu][e] = __builtin_fmaf(iu < split ? s[ju] : s1[ONE_SB ? 0 : ju], pring[u % PR][e], acc[ju][iu][e]);
                 asm volatile("" : "+v"(acc[ju][iu]));        // anchor: the fold happens in this slot
             } else {
                 const int u = NMFMA + t - LAG, ju = u / TN, iu = u % TN;   // tail of the previous K block
 #pragma unroll
-                for (int e = 0; e < 4; e++) acc[ju][iu][e] = __builtin_fmaf(s_last, pring[u % PR][e], acc[ju][iu][e]);
+                for (int e = 0; e < 4; e++)
+                    acc[ju][iu][e] = __builtin_fmaf(iu < split ? s_last : s1_last, pring[u % PR][e], acc[ju][iu][e]);
                 asm volatile("" : "+v"(acc[ju][iu]));
             }
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    int kb = kb_begin;
-    for (; kb + NS - 1 < kb_end; kb += NS) {
-        k_block(IntTag<0>{}, kb);
-        k_block(IntTag<1>{}, kb + 1);
-        if constexpr (NS > 2) k_block(IntTag<2 % NS>{}, kb + 2);
-        if constexpr (NS > 3) k_block(IntTag<3 % NS>{}, kb + 3);
-    }
-    if (kb < kb_end) k_block(IntTag<0>{}, kb);
-    if constexpr (NS > 2)
-        if (kb + 1 < kb_end) k_block(IntTag<1>{}, kb + 1);
-    if constexpr (NS > 3)
-        if (kb + 2 < kb_end) k_block(IntTag<2 % NS>{}, kb + 2);
-    // folds still owed by the last K block
+    auto k_loop = [&](auto split_c) {
+        constexpr int split = decltype(split_c)::value;
+        int kb = kb_begin;
+        for (; kb + 1 < kb_end; kb += 2) {
+            k_block(IntTag<0>{}, split_c, kb);
+            k_block(IntTag<1>{}, split_c, kb + 1);
+        }
+        if (kb < kb_end) k_block(IntTag<0>{}, split_c, kb);
+        // folds still owed by the last K block
 #pragma unroll
-    for (int t = 0; t < LAG; t++) {
-        const int u = NMFMA + t - LAG, ju = u / TN, iu = u % TN;
+        for (int t = 0; t < LAG; t++) {
+            const int u = NMFMA + t - LAG, ju = u / TN, iu = u % TN;
 #pragma unroll
-        for (int e = 0; e < 4; e++) acc[ju][iu][e] = __builtin_fmaf(s[TM - 1], pring[u % PR][e], acc[ju][iu][e]);
+            for (int e = 0; e < 4; e++)
+                acc[ju][iu][e] = __builtin_fmaf(iu < split ? s[TM - 1] : s1[ONE_SB ? 0 : TM - 1], pring[u % PR][e], acc[ju][iu][e]);
+        }
+    };
+    if constexpr (ONE_SB) {
+        k_loop(IntTag<TN>{});
+    } else {
+        // a wave whose columns lie in one block reads the same slot twice (sboff1 == sboff) and takes either path
+        if (sb_split == 1) k_loop(IntTag<1>{});
+        else k_loop(IntTag<2>{});
     }
     // LDS-DMA writes of the last (redundant) prefetches must land before this workgroup's LDS can be handed on
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -435,7 +498,10 @@ struct StoreGeom {
     static constexpr int REGION = ROWS * ROW;            // bytes per wave
     static_assert(G::TM % PASSES == 0, "whole m-tiles per pass");
 };
-template <int BM, int BN, int WAVES_M, int WAVES_N, int PASSES = 2, bool BARRIER = true>
+// Passes used when the staging overlays the stage buffers: the fewest that give whole store instructions.
+template <int BM, int WAVES_M>
+constexpr int default_store_passes() { return (BM / WAVES_M / 16) % 3 == 0 ? 3 : 2; }
+template <int BM, int BN, int WAVES_M, int WAVES_N, int PASSES = default_store_passes<BM, WAVES_M>(), bool BARRIER = true>
 __device__ __forceinline__ void store_tile_bf16(const f32x4 (&acc)[BM / WAVES_M / 16][BN / WAVES_N / 16],
                                                 uint16_t *__restrict__ C, int M, int N, int m0, int n0,
                                                 uint8_t *staging) {
@@ -443,9 +509,10 @@ __device__ __forceinline__ void store_tile_bf16(const f32x4 (&acc)[BM / WAVES_M 
     using S = StoreGeom<BM, BN, WAVES_M, WAVES_N, PASSES>;
     constexpr int ROW = S::ROW, ROWS = S::ROWS, TMP = G::TM / PASSES;
     constexpr int LPR = G::WN * 2 / 16;                  // lanes per row on the way out (16 bytes each)
-    constexpr int RPI = 64 / LPR;                        // rows per store instruction
+    constexpr bool WHOLE_ROWS = 64 % LPR == 0;           // a store instruction covers whole rows
+    constexpr int RPI = WHOLE_ROWS ? 64 / LPR : 1;       // rows per store instruction
     static_assert(!BARRIER || G::NW * S::REGION <= 2 * G::STAGE, "staging fits in the stage buffers");
-    static_assert(ROWS % RPI == 0, "whole store instructions");
+    static_assert(WHOLE_ROWS ? ROWS % RPI == 0 : (ROWS * LPR) % 64 == 0, "whole store instructions");
     // the opaque zero keeps this address arithmetic below the main loop: hoisted above it, it would cost the
     // loop dozens of registers
     int vz;
@@ -468,13 +535,25 @@ __device__ __forceinline__ void store_tile_bf16(const f32x4 (&acc)[BM / WAVES_M 
             }
         }
         // same wave writes and reads its region: program order is enough, the compiler inserts the LDS wait
+        if constexpr (WHOLE_ROWS) {
 #pragma unroll
-        for (int r0 = 0; r0 < ROWS; r0 += RPI) {
-            const int r = r0 + lane / LPR, cb = (lane % LPR) * 16;          // row in the pass, byte column
-            const uint4 v = *(const uint4 *)(region + r * ROW + cb);
-            const int m = m0 + wm * G::WM + h * ROWS + r;
-            const int n = n0 + wn * G::WN + cb / 2;
-            if (m < M && n < N) *(uint4 *)(C + (size_t)m * N + n) = v;
+            for (int r0 = 0; r0 < ROWS; r0 += RPI) {
+                const int r = r0 + lane / LPR, cb = (lane % LPR) * 16;          // row in the pass, byte column
+                const uint4 v = *(const uint4 *)(region + r * ROW + cb);
+                const int m = m0 + wm * G::WM + h * ROWS + r;
+                const int n = n0 + wn * G::WN + cb / 2;
+                if (m < M && n < N) *(uint4 *)(C + (size_t)m * N + n) = v;
+            }
+        } else {
+            // rows of LPR chunks with 64 % LPR != 0: the pass's chunks in row-major order, 64 per instruction
+#pragma unroll
+            for (int q0 = 0; q0 < ROWS * LPR; q0 += 64) {
+                const int q = q0 + lane, r = q / LPR, cb = (q % LPR) * 16;
+                const uint4 v = *(const uint4 *)(region + r * ROW + cb);
+                const int m = m0 + wm * G::WM + h * ROWS + r;
+                const int n = n0 + wn * G::WN + cb / 2;
+                if (m < M && n < N) *(uint4 *)(C + (size_t)m * N + n) = v;
+            }
         }
     }
 }
@@ -581,9 +660,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
     const int kb_end = kb_begin + kb_per_split < QK ? kb_begin + kb_per_split : QK;
     f32x4 acc[G::TM][G::TN];
     tile_mainloop<BM, BN, WAVES_M, WAVES_N, NS>(A, B, SA, SB, M, M, N, m0, n0, kb_begin, kb_end, lds, acc);
-    if constexpr (PARTIAL)
+    if constexpr (PARTIAL && 64 % (G::WN / 4) == 0)
         store_tile_f32_staged<BM, BN, WAVES_M, WAVES_N>(acc, (float *)Cout + ((size_t)blockIdx.y * M + m0) * N + n0, N,
                                                         M - m0, N - n0, lds);
+    else if constexpr (PARTIAL)
+        store_tile_f32<BM, BN, WAVES_M, WAVES_N>(acc, (float *)Cout + ((size_t)blockIdx.y * M + m0) * N + n0, N, M - m0,
+                                                 N - n0);
     else
         store_tile_bf16<BM, BN, WAVES_M, WAVES_N>(acc, (uint16_t *)Cout, M, N, m0, n0, lds);
 }
