@@ -278,6 +278,24 @@ def main():
                           "us": round(u, 2), "tflops": round(tf, 1), "pct_fp8_mfma_peak": round(100 * tf / PEAK_FP8_TFLOPS, 2)}
         print("grouped %s: %.2f us  %.1f TFLOP/s (%.1f %% of peak)" % (out["grouped"]["workload"], u, tf,
               100 * tf / PEAK_FP8_TFLOPS), file=sys.stderr)
+        # the same launch with other operand bits (same shapes, scales and plan): the chip's clock under load depends
+        # on how many bits toggle, so the time does too
+        out["operand_bits"] = {"quantised_normal_us": round(us, 2)}
+        for label in ("zeros", "random_bytes"):
+            ops = []
+            for t in g[:2]:
+                x = torch.empty_like(t)
+                u8 = x.view(torch.uint8)
+                if label == "zeros":
+                    u8.zero_()
+                else:
+                    u8.random_(0, 256)
+                    u8[(u8 & 0x7F) == 0x7F] = 0           # no NaN codes
+                ops.append(x)
+            u = time_gemm(rfk, [(ops[0], ops[1]) + tuple(g[2:])], args.steps, args.warmup, stream)
+            out["operand_bits"][label + "_us"] = round(u, 2)
+            del ops
+        print("C2 launch time by operand bits: %r" % (out["operand_bits"],), file=sys.stderr)
         # what the chip sustains on the same MFMA instruction from registers alone (clock under its power limit);
         # run as a child process once the GEMM work above is done
         probe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "radeonflow_kernels_amd", "lib", "mfma_ceiling")
