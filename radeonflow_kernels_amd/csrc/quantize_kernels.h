@@ -15,6 +15,7 @@
 namespace rf {
 
 template <int V> struct IntConst { static constexpr int value = V; };
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
 
 // fp32 -> OCP e4m3fn code, round to nearest even, anything that rounds above 448 (and NaN) becomes NaN (0x7F).
 // Integer/exact-float arithmetic only, so that it agrees bit for bit with a CPU implementation; no branches.
@@ -61,9 +62,31 @@ __global__ __launch_bounds__(256) void cast_f32_to_e4m3fn(const float *__restric
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __builtin_bit_cast(float, h << 16); }
 
-// Maximum over each aligned group of 16 lanes, left in all of them: four DPP steps (swap within pairs, within
-// quads, rotate the 16-lane row by 4 and by 8) instead of LDS-crossbar shuffles. x > a ? x : a, so a NaN never wins.
-__device__ __forceinline__ float max_over_16_lanes(float a) {
+// Maximum over each aligned group of 16 lanes, left in all of them, for N unsigned values at once: four DPP steps
+// (swap within pairs, within quads, rotate the 16-lane row by 4 and by 8) instead of LDS-crossbar shuffles, each one
+// v_max_u32 with a DPP operand. Written as asm because the compiler emits move + max for the builtin form. A DPP
+// operand must not be read within two instructions of the VALU write that produced it: the first step carries its
+// own wait, later steps of one value are N >= 3 volatile statements apart.
+template <int N>
+__device__ __forceinline__ void max_over_16_lanes(uint32_t (&a)[N]) {
+    static_assert(N >= 3, "steps of one value must be at least two instructions apart");
+#pragma unroll
+    for (int i = 0; i < N; i++)
+        asm volatile("s_nop 1\n\tv_max_u32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf" : "+v"(a[i]));
+#pragma unroll
+    for (int i = 0; i < N; i++)
+        asm volatile("v_max_u32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf" : "+v"(a[i]));
+#pragma unroll
+    for (int i = 0; i < N; i++)
+        asm volatile("v_max_u32_dpp %0, %0, %0 row_ror:4 row_mask:0xf bank_mask:0xf" : "+v"(a[i]));
+#pragma unroll
+    for (int i = 0; i < N; i++)
+        asm volatile("v_max_u32_dpp %0, %0, %0 row_ror:8 row_mask:0xf bank_mask:0xf" : "+v"(a[i]));
+    asm volatile("s_nop 1" ::: "memory");     // the compiler may follow up with a DPP or lane-crossing read of a[N-1]
+}
+
+// The same for one float with "a NaN never wins" comparisons (the rare path of rows that contain a NaN).
+__device__ __forceinline__ float max_over_16_lanes_nan_safe(float a) {
     auto step = [&](auto ctrl) {
         const float o = __builtin_bit_cast(
             float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, a), decltype(ctrl)::value, 0xf, 0xf, false));
@@ -74,6 +97,16 @@ __device__ __forceinline__ float max_over_16_lanes(float a) {
     step(IntConst<0x124>{});     // row_ror 4
     step(IntConst<0x128>{});     // row_ror 8
     return a;
+}
+
+// a / 448 for a in [2^-100, FLT_MAX]: product with RN(1/448) plus one correction step through the exact remainder.
+// Compared with the IEEE division over every float in that range on the CPU: identical (below 2^-100 the remainder
+// underflows and it is not).
+__device__ __forceinline__ float div_by_448(float a) {
+    constexpr float C = 1.0f / 448.0f;
+    const float q = a * C;
+    const float r = __builtin_fmaf(-q, 448.0f, a);
+    return __builtin_fmaf(r, C, q);
 }
 
 // One workgroup (256 threads) per 128 x 128 block: rows r0.. of X (ld = K elements), K block kb.
@@ -94,51 +127,84 @@ __global__ __launch_bounds__(256) void quantize_block128(const void *__restrict_
     auto row_of = [&](int i) { return (i >> 2) * (128 / NG) + 4 * rsub + (i & 3); };
     // K blocks vary fastest over the grid: workgroups that run together read neighbouring pieces of the same rows
     const int rb = blockIdx.y, r0 = rb * 128, kb = blockIdx.x, k0 = kb * 128;
+    // All loads are issued before the first one is used: rows past R read row R-1 again (their results are never
+    // stored, and they are kept out of a block-wide maximum below) instead of sitting behind a branch each.
+    uint4 raw[RPT];
+#pragma unroll
+    for (int i = 0; i < RPT; i++) {
+        const int r = r0 + row_of(i), rc = r < R ? r : R - 1;
+        const size_t off = (size_t)rc * K + k0 + KPT * lane_k;
+        raw[i] = IN_BF16 ? *(const uint4 *)((const uint16_t *)X + off) : *(const uint4 *)((const float *)X + off);
+    }
     float v[RPT][KPT];
 #pragma unroll
     for (int i = 0; i < RPT; i++) {
-        const int r = r0 + row_of(i);
-        if (r < R) {
+        const uint32_t q[4] = {raw[i].x, raw[i].y, raw[i].z, raw[i].w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
             if constexpr (IN_BF16) {
-                const uint4 w = *(const uint4 *)((const uint16_t *)X + (size_t)r * K + k0 + KPT * lane_k);
-                const uint32_t q[4] = {w.x, w.y, w.z, w.w};
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    v[i][2 * e] = bf16_bits_to_f32(q[e] & 0xffffu);
-                    v[i][2 * e + 1] = bf16_bits_to_f32(q[e] >> 16);
-                }
+                v[i][2 * e] = bf16_bits_to_f32(q[e] & 0xffffu);
+                v[i][2 * e + 1] = bf16_bits_to_f32(q[e] >> 16);
             } else {
-                const float4 w = *(const float4 *)((const float *)X + (size_t)r * K + k0 + KPT * lane_k);
-                v[i][0] = w.x; v[i][1] = w.y; v[i][2] = w.z; v[i][3] = w.w;
+                v[i][e] = __builtin_bit_cast(float, q[e]);
             }
-        } else {
-#pragma unroll
-            for (int e = 0; e < KPT; e++) v[i][e] = 0.f;
         }
     }
-    // amax: NaNs never win a comparison, like a scalar "if (|x| > amax)" loop
-    float amax[RPT];
+    // amax: NaNs never win a comparison, like a scalar "if (|x| > amax)" loop. For everything but NaNs the order of
+    // |x| is the order of its bit pattern as an unsigned integer, and NaN patterns lie above infinity: the maximum is
+    // taken on the raw bits (two bf16 per instruction), and a row whose maximum lands above infinity contains a NaN
+    // and takes the comparison loop instead.
+    uint32_t amax_bits[RPT];
 #pragma unroll
     for (int i = 0; i < RPT; i++) {
-        float a = 0.f;
+        const uint32_t q[4] = {raw[i].x, raw[i].y, raw[i].z, raw[i].w};
+        if constexpr (IN_BF16) {
+            u16x2 m = {0, 0};
 #pragma unroll
-        for (int e = 0; e < KPT; e++) { const float x = __builtin_fabsf(v[i][e]); a = x > a ? x : a; }
-        a = max_over_16_lanes(a);
-        if constexpr (LPR == 32) { const float o = __shfl_xor(a, 16, 64); a = o > a ? o : a; }
-        amax[i] = a;                                          // all LPR lanes of the row hold it
+            for (int e = 0; e < 4; e++) m = __builtin_elementwise_max(m, __builtin_bit_cast(u16x2, q[e] & 0x7fff7fffu));
+            amax_bits[i] = (uint32_t)(m[0] > m[1] ? m[0] : m[1]) << 16;
+        } else {
+            uint32_t m = 0;
+#pragma unroll
+            for (int e = 0; e < 4; e++) { const uint32_t x = q[e] & 0x7fffffffu; m = x > m ? x : m; }
+            amax_bits[i] = m;
+        }
     }
+    max_over_16_lanes(amax_bits);                             // all 16 lanes of a row group hold it
+    float amax[RPT];
+    bool has_nan[RPT];
+#pragma unroll
+    for (int i = 0; i < RPT; i++) {
+        if constexpr (LPR == 32) { const uint32_t o = __shfl_xor(amax_bits[i], 16, 64); amax_bits[i] = o > amax_bits[i] ? o : amax_bits[i]; }
+        amax[i] = __builtin_bit_cast(float, amax_bits[i]);
+        has_nan[i] = amax_bits[i] > 0x7f800000u;              // the same in all lanes of the row
+        if (__builtin_expect(has_nan[i], 0)) {
+            float a = 0.f;
+#pragma unroll
+            for (int e = 0; e < KPT; e++) { const float x = __builtin_fabsf(v[i][e]); a = x > a ? x : a; }
+            a = max_over_16_lanes_nan_safe(a);
+            if constexpr (LPR == 32) { const float o = __shfl_xor(a, 16, 64); a = o > a ? o : a; }
+            amax[i] = a;
+        }
+    }
+    // scale = amax / 448, exactly as the IEEE division gives it
+    auto scale_of = [](float a) {
+        float sc = a > 0.f ? div_by_448(a) : 1.0f;
+        if (__builtin_expect(a > 0.f && !(a >= 0x1p-100f && a <= 0x1.fffffep127f), 0)) sc = a / 448.0f;
+        return sc;
+    };
     float s[RPT];
     if constexpr (PER_ROW) {
 #pragma unroll
         for (int i = 0; i < RPT; i++) {
-            s[i] = amax[i] > 0.f ? amax[i] / 448.0f : 1.0f;
+            s[i] = scale_of(amax[i]);
             const int r = r0 + row_of(i);
             if (lane_k == 0 && r < R) scales[(size_t)kb * scale_ld + r] = s[i];
         }
     } else {
         float a = 0.f;
 #pragma unroll
-        for (int i = 0; i < RPT; i++) a = amax[i] > a ? amax[i] : a;
+        for (int i = 0; i < RPT; i++) a = (amax[i] > a && r0 + row_of(i) < R) ? amax[i] : a;
 #pragma unroll
         for (int off = LPR; off < 64; off <<= 1) { const float o = __shfl_xor(a, off, 64); a = o > a ? o : a; }
         if ((t & 63) == 0) wave_max[t >> 6] = a;
@@ -146,42 +212,52 @@ __global__ __launch_bounds__(256) void quantize_block128(const void *__restrict_
         a = wave_max[0];
 #pragma unroll
         for (int w = 1; w < 4; w++) a = wave_max[w] > a ? wave_max[w] : a;
-        const float sb = a > 0.f ? a / 448.0f : 1.0f;
+        const float sb = scale_of(a);
 #pragma unroll
         for (int i = 0; i < RPT; i++) s[i] = sb;
         if (t == 0) scales[(size_t)kb * scale_ld + rb] = sb;
     }
     // quantise and transpose through LDS: tile[k][row]. The value to encode is fl32(x / scale). A correctly rounded
-    // division costs ~15 instructions; instead y = x * (1 / scale) is used, which is within 2^-22 (relative) of that
-    // quotient. The fp8 conversion is monotonic, so if y * (1 - 2^-21) and y * (1 + 2^-21) convert to the same code,
-    // the exact quotient (which lies between them) converts to that code too. Only when the two differ (a rounding
-    // boundary is that close: about 1 element in 10^5), or a NaN is involved, or the scale is so far from 1 that its
-    // reciprocal is not a normal number, the group of four is redone with the division.
-    float rinv[RPT];
-    bool fast[RPT];
+    // division costs ~11 instructions per element. Instead, with r = rcp(scale) (the hardware reciprocal, within a few
+    // ulp of 1 / scale), x * (r * (1 + 2^-20)) and x * (r * (1 - 2^-20)) are, in magnitude, above and below the exact
+    // quotient and its fp32 rounding (the factors' rounding errors and the reciprocal's error are below 2^-21
+    // together). The fp8 conversion is monotonic, so if the two products convert to the same code, fl32(x / scale)
+    // converts to that code too. Only when they differ (a rounding boundary is that close: about 1 element in 10^5),
+    // or the row contains a NaN, or the scale is so far from 1 that its reciprocal is not a normal number, the group of
+    // four is redone with the division.
+    float rup[RPT], rdown[RPT];
+    bool fast[RPT / 4];
 #pragma unroll
     for (int i = 0; i < RPT; i++) {
-        rinv[i] = 1.0f / s[i];
-        fast[i] = s[i] > 0x1p-100f && s[i] < 0x1p100f;
+        const float rinv = __builtin_amdgcn_rcpf(s[i]);
+        rup[i] = rinv * (1.0f + 0x1p-20f);
+        rdown[i] = rinv * (1.0f - 0x1p-20f);
+    }
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+        fast[g] = true;
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            fast[g] = fast[g] && s[4 * g + j] > 0x1p-100f && s[4 * g + j] < 0x1p100f && !has_nan[4 * g + j];
     }
 #pragma unroll
     for (int g = 0; g < NG; g++)
 #pragma unroll
         for (int e = 0; e < KPT; e++) {
-            float y[4];
-            bool ok = true;
+            float yu[4], yd[4];
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                y[j] = v[4 * g + j][e] * rinv[4 * g + j];
-                ok = ok && fast[4 * g + j] && y[j] == y[j];
+                yu[j] = v[4 * g + j][e] * rup[4 * g + j];
+                yd[j] = v[4 * g + j][e] * rdown[4 * g + j];
             }
-            constexpr float UP = 1.0f + 0x1p-21f, DOWN = 1.0f - 0x1p-21f;
-            int hi = __builtin_amdgcn_cvt_pk_fp8_f32(y[0] * UP, y[1] * UP, 0, false);
-            hi = __builtin_amdgcn_cvt_pk_fp8_f32(y[2] * UP, y[3] * UP, hi, true);
-            int lo = __builtin_amdgcn_cvt_pk_fp8_f32(y[0] * DOWN, y[1] * DOWN, 0, false);
-            lo = __builtin_amdgcn_cvt_pk_fp8_f32(y[2] * DOWN, y[3] * DOWN, lo, true);
+            // (the first conversion of a word keeps the upper half of its old value, which the second one overwrites:
+            // any register will do as the old value)
+            int hi = __builtin_amdgcn_cvt_pk_fp8_f32(yu[0], yu[1], __builtin_bit_cast(int, yu[0]), false);
+            hi = __builtin_amdgcn_cvt_pk_fp8_f32(yu[2], yu[3], hi, true);
+            int lo = __builtin_amdgcn_cvt_pk_fp8_f32(yd[0], yd[1], __builtin_bit_cast(int, yd[0]), false);
+            lo = __builtin_amdgcn_cvt_pk_fp8_f32(yd[2], yd[3], lo, true);
             uint32_t w = (uint32_t)hi;
-            if (!ok || hi != lo)
+            if (!fast[g] || hi != lo)
                 w = f32x4_to_e4m3fn_codes(v[4 * g][e] / s[4 * g], v[4 * g + 1][e] / s[4 * g + 1],
                                           v[4 * g + 2][e] / s[4 * g + 2], v[4 * g + 3][e] / s[4 * g + 3]);
             *(uint32_t *)(tile + (KPT * lane_k + e) * PITCH + row_of(4 * g)) = w;
