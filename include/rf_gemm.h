@@ -106,7 +106,8 @@ void rf_gemm_destroy(void);
  *                row_offsets[g] .. row_offsets[g+1]-1 (empty groups allowed); read before the call returns.
  * groups <= 256. Offsets that are all multiples of 16 (with N % 16 == 0 and 16-byte aligned a, b, c) take the tiled
  * kernel in one launch; anything else runs the bounds-checked kernel once per group.
- * variant: -1 = automatic, else an index into {256x256, 128x256, 128x128, 128x64} tiles. */
+ * variant: -1 = automatic, else an index into {256x256, 128x256, 128x128, 128x64} tiles, or 4 = 256-row tiles with a
+ * 128 x 256 tile for a group's last rows when at most 128 are left. */
 int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const float *bs, void *c, const int *row_offsets,
                         int groups, int n, int k, int variant, hipStream_t stream);
 

@@ -792,6 +792,43 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_gro
     store_tile_bf16<BM, BN, WAVES_M, WAVES_N>(acc, C + (size_t)row0 * N, rows, N, m0, n0, lds);
 }
 
+// The same with two tile heights in one launch: a group's rows are cut into 256-row tiles, and what is left over
+// goes to a 128 x 256 tile when it is at most 128 rows (otherwise to one more 256-row tile). With uneven groups half
+// of the left-overs are that small, and a 128-row tile costs little more than half a 256-row one. tile_start counts
+// a group's workgroups: first its 256-row tiles, then the columns of its 128-row tile. Both paths are 8 waves and
+// share the LDS allocation; the branch is uniform over the workgroup.
+__global__ __launch_bounds__(512) void gemm_fp8_blockscale_grouped_mixed(
+    const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
+    const float *__restrict__ SB, uint16_t *__restrict__ C, int M_total, int N, int K, int groups, int tiles_n,
+    int group_m, const GroupTable table) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    int lo = 0, hi = groups;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (table.tile_start[mid] <= (int)blockIdx.x) lo = mid; else hi = mid;
+    }
+    const int grp = lo, row0 = table.row_start[grp], rows = table.row_start[grp + 1] - row0;
+    const int local = blockIdx.x - table.tile_start[grp];
+    const int big_m = rows / 256 + (rows % 256 > 128 ? 1 : 0);       // 256-row tiles of this group
+    const int QK = K / BK, QN = (N + 127) / 128;
+    const uint8_t *Bg = B + (size_t)grp * K * N;
+    const float *SBg = SB + (size_t)grp * QK * QN;
+    if (local < big_m * tiles_n) {
+        int tile_m, tile_n;
+        tile_of_block(local, big_m * tiles_n, big_m, tiles_n, group_m, false, tile_m, tile_n);
+        const int m0 = tile_m * 256, n0 = tile_n * 256;
+        f32x4 acc[TileGeom<256, 256, 2, 4>::TM][TileGeom<256, 256, 2, 4>::TN];
+        tile_mainloop<256, 256, 2, 4>(A + row0, Bg, SA + row0, SBg, rows, M_total, N, m0, n0, 0, QK, lds, acc);
+        store_tile_bf16<256, 256, 2, 4>(acc, C + (size_t)row0 * N, rows, N, m0, n0, lds);
+    } else {
+        const int r1 = row0 + big_m * 256, rest = rows - big_m * 256;  // 16..128 rows
+        const int n0 = (local - big_m * tiles_n) * 256;
+        f32x4 acc[TileGeom<128, 256, 2, 4>::TM][TileGeom<128, 256, 2, 4>::TN];
+        tile_mainloop<128, 256, 2, 4>(A + r1, Bg, SA + r1, SBg, rest, M_total, N, 0, n0, 0, QK, lds, acc);
+        store_tile_bf16<128, 256, 2, 4>(acc, C + (size_t)r1 * N, rest, N, 0, n0, lds);
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // Bounds-checked kernel for shapes or alignments the tiled kernel does not take (M or N not a
 // multiple of 16, unaligned pointers). One wave per 16x16 output tile, bytes gathered directly

@@ -55,13 +55,14 @@ def _check_canary(buf, used):
 
 
 CASES = [([256, 128, 512, 64], 512, 256), ([16, 0, 48, 400, 0, 32], 576, 384), ([1024], 256, 512),
-         ([128] * 32, 2048, 256), ([0, 0, 272], 144, 128), ([640, 16, 16, 2048, 112], 7168, 256)]
+         ([128] * 32, 2048, 256), ([0, 0, 272], 144, 128), ([640, 16, 16, 2048, 112], 7168, 256),
+         ([272, 384, 128, 400, 16, 656], 512, 256)]      # left-overs of 16, 128, 128, 144, 16 and 144 rows
 
 
 @pytest.mark.parametrize("rows,n,k", CASES)
 def test_grouped_bit_exact_on_exact_data(rfk, rows, n, k):
     g, offs, exp = _grouped_problem(rows, n, k, seed=11 * n + k, exact=True)
-    for variant in (-1, 0, 1, 2, 3):
+    for variant in (-1, 0, 1, 2, 3, 4):
         g[4].zero_()
         rfk.fp8_mm_grouped(*g[:5], offs, variant=variant)
         torch.cuda.synchronize()
