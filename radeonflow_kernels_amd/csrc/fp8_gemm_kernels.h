@@ -312,7 +312,7 @@ __device__ __forceinline__ void tile_mainloop(
     //     per slot, and run on into the first slots of the next iteration.
     // An empty volatile asm after each MFMA / fold anchors it in its slot, sched_barrier(0) keeps the slots apart;
     // the compiler still places the LDS waits and hazard nops.
-    constexpr int NMFMA = TM * TN, PR = NMFMA % 4 == 0 ? 4 : 3, LAG = PR - 1, BAR_SLOT = (TM - 1) * TN;
+    constexpr int NMFMA = TM * TN, PR = (NMFMA % 4 == 0 && TN > 3) ? 4 : 3, LAG = PR - 1, BAR_SLOT = (TM - 1) * TN;
     static_assert(NMFMA % PR == 0, "ring positions repeat per K block");
     static_assert(LAG < TN && LAG < PR, "lagged folds of a K block stay inside its last m-tile row");
     static_assert(TM % 2 == 0, "the last m-tile uses afrag[1], so afrag[0] is free for the next block");
@@ -587,8 +587,10 @@ __device__ __forceinline__ void store_tile_f32_staged(const f32x4 (&acc)[BM / WA
                                                       uint8_t *staging) {
     using G = TileGeom<BM, BN, WAVES_M, WAVES_N>;
     constexpr int ROW = G::WN * 4 + 16, REGION = 16 * ROW;
-    constexpr int LPR = G::WN / 4, RPI = 64 / LPR;        // lanes per row (16 bytes each), rows per store instruction
-    static_assert(G::NW * REGION <= 2 * G::STAGE && 64 % LPR == 0 && 16 % RPI == 0, "staging geometry");
+    constexpr int LPR = G::WN / 4;                        // lanes per row (16 bytes each)
+    constexpr bool WHOLE_ROWS = 64 % LPR == 0;            // a store instruction covers whole rows
+    constexpr int RPI = WHOLE_ROWS ? 64 / LPR : 1;        // rows per store instruction
+    static_assert(G::NW * REGION <= 2 * G::STAGE && (WHOLE_ROWS ? 16 % RPI == 0 : (16 * LPR) % 64 == 0), "staging geometry");
     int vz;                                  // see store_tile_bf16
     asm volatile("v_mov_b32 %0, 0" : "=v"(vz));
     const int lane = (threadIdx.x & 63) + vz, wave = threadIdx.x >> 6, L = lane & 15, g = lane >> 4;
@@ -599,12 +601,23 @@ __device__ __forceinline__ void store_tile_f32_staged(const f32x4 (&acc)[BM / WA
     for (int j = 0; j < G::TM; j++) {
 #pragma unroll
         for (int i = 0; i < G::TN; i++) *(f32x4 *)(region + L * ROW + (16 * i + 4 * g) * 4) = acc[j][i];
+        if constexpr (WHOLE_ROWS) {
 #pragma unroll
-        for (int r0 = 0; r0 < 16; r0 += RPI) {
-            const int r = r0 + lane / LPR, cb = (lane % LPR) * 16;
-            const uint4 v = *(const uint4 *)(region + r * ROW + cb);
-            const int m = wm * G::WM + 16 * j + r, n = wn * G::WN + cb / 4;
-            if (m < m_lim && n < n_lim) *(uint4 *)(t + (size_t)m * ld + n) = v;
+            for (int r0 = 0; r0 < 16; r0 += RPI) {
+                const int r = r0 + lane / LPR, cb = (lane % LPR) * 16;
+                const uint4 v = *(const uint4 *)(region + r * ROW + cb);
+                const int m = wm * G::WM + 16 * j + r, n = wn * G::WN + cb / 4;
+                if (m < m_lim && n < n_lim) *(uint4 *)(t + (size_t)m * ld + n) = v;
+            }
+        } else {
+            // rows of LPR chunks with 64 % LPR != 0: the m-tile's chunks in row-major order, 64 per instruction
+#pragma unroll
+            for (int q0 = 0; q0 < 16 * LPR; q0 += 64) {
+                const int q = q0 + lane, r = q / LPR, cb = (q % LPR) * 16;
+                const uint4 v = *(const uint4 *)(region + r * ROW + cb);
+                const int m = wm * G::WM + 16 * j + r, n = wn * G::WN + cb / 4;
+                if (m < m_lim && n < n_lim) *(uint4 *)(t + (size_t)m * ld + n) = v;
+            }
         }
     }
 }
@@ -660,12 +673,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
     const int kb_end = kb_begin + kb_per_split < QK ? kb_begin + kb_per_split : QK;
     f32x4 acc[G::TM][G::TN];
     tile_mainloop<BM, BN, WAVES_M, WAVES_N, NS>(A, B, SA, SB, M, M, N, m0, n0, kb_begin, kb_end, lds, acc);
-    if constexpr (PARTIAL && 64 % (G::WN / 4) == 0)
+    if constexpr (PARTIAL)
         store_tile_f32_staged<BM, BN, WAVES_M, WAVES_N>(acc, (float *)Cout + ((size_t)blockIdx.y * M + m0) * N + n0, N,
                                                         M - m0, N - n0, lds);
-    else if constexpr (PARTIAL)
-        store_tile_f32<BM, BN, WAVES_M, WAVES_N>(acc, (float *)Cout + ((size_t)blockIdx.y * M + m0) * N + n0, N, M - m0,
-                                                 N - n0);
     else
         store_tile_bf16<BM, BN, WAVES_M, WAVES_N>(acc, (uint16_t *)Cout, M, N, m0, n0, lds);
 }
