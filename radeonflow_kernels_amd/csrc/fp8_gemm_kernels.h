@@ -559,28 +559,9 @@ __device__ __forceinline__ void store_tile_bf16(const f32x4 (&acc)[BM / WAVES_M 
 }
 
 // fp32 tile with leading dimension ld; rows < m_lim and cols < n_lim are written (limits relative to the tile).
-template <int BM, int BN, int WAVES_M, int WAVES_N>
-__device__ __forceinline__ void store_tile_f32(const f32x4 (&acc)[BM / WAVES_M / 16][BN / WAVES_N / 16],
-                                               float *__restrict__ t, size_t ld, int m_lim, int n_lim) {
-    using G = TileGeom<BM, BN, WAVES_M, WAVES_N>;
-    int vz;                                  // see store_tile_bf16
-    asm volatile("v_mov_b32 %0, 0" : "=v"(vz));
-    const int lane = (threadIdx.x & 63) + vz, wave = threadIdx.x >> 6, L = lane & 15, g = lane >> 4;
-    const int wm = wave % WAVES_M, wn = wave / WAVES_M;
-#pragma unroll
-    for (int j = 0; j < G::TM; j++) {
-        const int m = wm * G::WM + 16 * j + L;
-#pragma unroll
-        for (int i = 0; i < G::TN; i++) {
-            const int n = wn * G::WN + 16 * i + 4 * g;
-            if (m < m_lim && n < n_lim) *(f32x4 *)(t + (size_t)m * ld + n) = acc[j][i];
-        }
-    }
-}
-
-// The same through LDS, one m-tile (16 rows) of every wave per pass, written out 16 bytes per lane with neighbouring
-// lanes along a row: each store instruction covers whole rows of the wave tile (256 contiguous bytes for 64 columns)
-// instead of sixteen 64-byte pieces. Starts with a barrier like store_tile_bf16 (the regions overlay the stages).
+// Through LDS, one m-tile (16 rows) of every wave per pass, written out 16 bytes per lane with neighbouring lanes along
+// a row: each store instruction covers whole rows of the wave tile (256 contiguous bytes for 64 columns) instead of
+// sixteen 64-byte pieces. Starts with a barrier like store_tile_bf16 (the regions overlay the stages).
 template <int BM, int BN, int WAVES_M, int WAVES_N>
 __device__ __forceinline__ void store_tile_f32_staged(const f32x4 (&acc)[BM / WAVES_M / 16][BN / WAVES_N / 16],
                                                       float *__restrict__ t, size_t ld, int m_lim, int n_lim,

@@ -15,7 +15,6 @@
 
 #include "../../include/rf_gemm.h"
 #include "fp8_gemm_kernels.h"
-#include "fp8_gemm_hold_a.h"
 #include "fp8_gemm_persistent.h"
 #include "quantize_kernels.h"
 
@@ -62,20 +61,14 @@ struct Variant {
     Variant { BM, BN, WM, WN, rf::TileGeom<BM, BN, WM, WN>::LDS_BYTES,                     \
               rf::gemm_fp8_blockscale_tile<BM, BN, WM, WN, false>,                         \
               rf::gemm_fp8_blockscale_tile<BM, BN, WM, WN, true>, nullptr, nullptr, 0 }
-// tiles with sides that are not powers of two (A fragments held, B streamed)
-#define RF_VARIANT_HOLD_A(BM, BN, WM, WN)                                                  \
-    Variant { BM, BN, WM, WN, rf::HoldAGeom<BM, BN, WM, WN>::LDS_BYTES,                    \
-              rf::gemm_fp8_blockscale_tile_hold_a<BM, BN, WM, WN, false>,                  \
-              rf::gemm_fp8_blockscale_tile_hold_a<BM, BN, WM, WN, true>, nullptr, nullptr, 0 }
 const Variant kVariants[] = {
     RF_VARIANT(256, 256, 2, 4),   // 0: 8 waves, wave tile 128(m) x 64(n), 128 KiB LDS
     RF_VARIANT(128, 128, 2, 2),   // 1: 4 waves, wave tile 64 x 64, 64 KiB LDS (2 workgroups per CU)
     RF_VARIANT(256, 128, 2, 2),   // 2: 4 waves, wave tile 128 x 64, 96 KiB LDS
     RF_VARIANT(128, 256, 2, 4),   // 3: 8 waves, wave tile 64 x 64, 96 KiB LDS
     RF_VARIANT(128, 64, 2, 1),    // 4: 2 waves, wave tile 64 x 64, 48 KiB LDS (3 workgroups per CU)
-    RF_VARIANT_HOLD_A(192, 288, 4, 2),   // 5: 8 waves, wave tile 48 x 144, 122 KiB LDS (6144 x 4608 = 512 tiles)
-    RF_VARIANT_TILE_ONLY(192, 192, 2, 4),   // 6: 8 waves, wave tile 96 x 48, 98 KiB LDS (6144 x 4608 = 768 tiles = 3 x 256)
-    RF_VARIANT_TILE_ONLY(128, 192, 2, 4),   // 7: 8 waves, wave tile 64 x 48, 82 KiB LDS (N = 576, 1536: no padded columns)
+    RF_VARIANT_TILE_ONLY(192, 192, 2, 4),   // 5: 8 waves, wave tile 96 x 48, 98 KiB LDS (6144 x 4608 = 768 tiles = 3 x 256)
+    RF_VARIANT_TILE_ONLY(128, 192, 2, 4),   // 6: 8 waves, wave tile 64 x 48, 82 KiB LDS (N = 576, 1536: no padded columns)
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
@@ -190,7 +183,7 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, rf_gemm_confi
     // win where they divide the shape into fuller rounds or leave no padded columns, e.g. N = 576, 1536 or 3072); the
     // smaller ones never won by more than a few percent.
     struct Candidate { int variant; double c, f; };
-    const Candidate cands[] = {{0, 1.355, 9.46}, {3, 0.769, 3.61}, {6, 0.95, 6.0}, {7, 0.65, 4.0}};
+    const Candidate cands[] = {{0, 1.355, 9.46}, {3, 0.769, 3.61}, {5, 0.95, 6.0}, {6, 0.65, 4.0}};
     const double f_next = 3.61, reduce_fixed = 6.83, reduce_per_elem = 8.7e-7;
     const int splits_tried[] = {1, 2, 3, 4, 6, 8, 12, 16};
     const int qk = k / rf::BK;
