@@ -77,6 +77,17 @@ int rf_fp8_gemm_ex(const void *a, const void *b, const float *as, const float *b
  * per-shape table in src/gemm/gemm_launcher.cpp:229-259 / tuner/gemm_tuner.py. */
 int rf_gemm_select_config(int m, int n, int k, rf_gemm_config *out);
 
+/* Measured plans from a file, looked up before the built-in table (the role of pasting DISPATCH_GEMM lines into the
+ * reference's launcher, src/gemm/gemm_launcher.cpp:229-259, tuner/gemm_batch.py:196-200, without a rebuild). One plan
+ * per line: "M N K variant split_k group_m stream_k"; braces and commas are blanks, '#' and "//" start a comment, so
+ * the tuner's --emit-file output and csrc/tuned_plans.inc are both valid files. *count receives the number of plans
+ * added (may be NULL). A line that does not parse or names a variant or schedule that does not exist fails the whole
+ * file with RF_ERR_BAD_CONFIG (nothing is added). A plan that cannot run for its shape (e.g. the persistent schedule on
+ * a ragged shape) is skipped at lookup. The file named by the environment variable RF_GEMM_PLANS is loaded the same
+ * way before the first plan is chosen. rf_gemm_clear_plans forgets all loaded plans. */
+int rf_gemm_load_plans(const char *path, int *count);
+void rf_gemm_clear_plans(void);
+
 /* Variant table introspection (for the tuner and tests). Returns RF_ERR_BAD_CONFIG past the end. */
 int rf_gemm_num_variants(void);
 int rf_gemm_variant_info(int variant, int *block_m, int *block_n, int *waves_m, int *waves_n, int *lds_bytes);

@@ -73,8 +73,14 @@ const Variant kVariants[] = {
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
 // ---- process-wide state ---------------------------------------------------------------------
+struct TunedPlan {
+    int m, n, k, variant, split_k, group_m, stream_k;
+};
+
 struct State {
     std::mutex mu;
+    std::vector<TunedPlan> user_plans;   // rf_gemm_load_plans / RF_GEMM_PLANS: looked up before the built-in table
+    bool env_plans_checked = false;
     float *ws = nullptr;
     size_t ws_bytes = 0;
     unsigned *tile_count = nullptr;      // stream-K arrival counters, zero between launches
@@ -87,8 +93,49 @@ State &state() {
     return s;
 }
 
+// Plan file: one plan per line, "M N K variant split_k group_m stream_k"; braces and commas count as blanks (so a
+// tuned_plans.inc written by the tuner is a plan file too), '#' and "//" start a comment. Appends to `out`.
+int parse_plans(const char *path, std::vector<TunedPlan> &out) {
+    FILE *f = fopen(path, "r");
+    if (!f) return fail(RF_ERR_BAD_CONFIG, std::string("cannot open plan file ") + path);
+    char line[512];
+    int lineno = 0;
+    std::vector<TunedPlan> plans;
+    while (fgets(line, sizeof line, f)) {
+        lineno++;
+        if (char *c = strstr(line, "//")) *c = 0;
+        if (char *c = strchr(line, '#')) *c = 0;
+        for (char *c = line; *c; c++)
+            if (*c == '{' || *c == '}' || *c == ',') *c = ' ';
+        TunedPlan p;
+        char extra;
+        const int got = sscanf(line, " %d %d %d %d %d %d %d %c", &p.m, &p.n, &p.k, &p.variant, &p.split_k, &p.group_m,
+                               &p.stream_k, &extra);
+        if (got <= 0) continue;                       // blank or comment line
+        if (got != 7 || p.m < 1 || p.n < 1 || p.k < rf::BK || p.k % rf::BK != 0 || p.variant < 0 ||
+            p.variant >= kNumVariants || p.split_k < 1 || p.group_m < 1 || p.stream_k < RF_SCHEDULE_TILES ||
+            p.stream_k > RF_SCHEDULE_PERSISTENT || (p.stream_k != RF_SCHEDULE_TILES && p.split_k != 1)) {
+            fclose(f);
+            return fail(RF_ERR_BAD_CONFIG, std::string(path) + ":" + std::to_string(lineno) +
+                                               ": expected \"M N K variant split_k group_m stream_k\" with valid values");
+        }
+        plans.push_back(p);
+    }
+    fclose(f);
+    out.insert(out.end(), plans.begin(), plans.end());
+    return RF_OK;
+}
+
 int ensure_device_info(State &s) {
     if (s.attrs_set) return RF_OK;
+    if (!s.env_plans_checked) {
+        // a file named by RF_GEMM_PLANS is loaded once, before the first plan is chosen; a bad file is an error
+        if (const char *path = getenv("RF_GEMM_PLANS")) {
+            int rc = parse_plans(path, s.user_plans);
+            if (rc != RF_OK) return rc;
+        }
+        s.env_plans_checked = true;
+    }
     int dev = 0;
     RF_HIP(hipGetDevice(&dev));
     hipDeviceProp_t prop;
@@ -148,16 +195,14 @@ bool persistent_ok(const Variant &v, int m, int n, int k) {
 // Plans measured on one MI355X by the tuner (python -m radeonflow_kernels_amd.tuner.gemm_tuner --all --emit).
 // The role of the reference's DISPATCH_GEMM table (src/gemm/gemm_launcher.cpp:229-259), except that a shape
 // outside the table is not an error: it gets the heuristic below.
-struct TunedPlan {
-    int m, n, k, variant, split_k, group_m, stream_k;
-};
 const TunedPlan kTunedPlans[] = {
     {0, 0, 0, 0, 1, 1, 0},
 #include "tuned_plans.inc"
 };
 
 // Heuristic plan for shapes without a measured entry. Inputs: shape and CU count.
-void select_config(int m, int n, int k, int num_cu, bool tiled_ok, rf_gemm_config *out) {
+void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::vector<TunedPlan> &user_plans,
+                   rf_gemm_config *out) {
     out->split_k = 1;
     out->group_m = 8;
     out->stream_k = 0;
@@ -165,15 +210,23 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, rf_gemm_confi
         out->variant = -1;
         return;
     }
+    auto usable = [&](const TunedPlan &p) {
+        return p.m == m && p.n == n && p.k == k && p.variant < kNumVariants && p.split_k <= k / rf::BK &&
+               (p.stream_k != RF_SCHEDULE_PERSISTENT || persistent_ok(kVariants[p.variant], m, n, k)) &&
+               (p.stream_k != RF_SCHEDULE_STREAM_K || kVariants[p.variant].streamk);
+    };
+    const TunedPlan *hit = nullptr;
+    for (const TunedPlan &p : user_plans)
+        if (!hit && usable(p)) hit = &p;
     for (const TunedPlan &p : kTunedPlans)
-        if (p.m == m && p.n == n && p.k == k && p.variant < kNumVariants && p.split_k <= k / rf::BK &&
-            (p.stream_k != RF_SCHEDULE_PERSISTENT || persistent_ok(kVariants[p.variant], m, n, k))) {
-            out->variant = p.variant;
-            out->split_k = p.split_k;
-            out->group_m = p.group_m;
-            out->stream_k = p.stream_k;
-            return;
-        }
+        if (!hit && usable(p)) hit = &p;
+    if (hit) {
+        out->variant = hit->variant;
+        out->split_k = hit->split_k;
+        out->group_m = hit->group_m;
+        out->stream_k = hit->stream_k;
+        return;
+    }
     // No measured entry: a cost model fitted to the tuner's measurements of the tabled shapes (it lands within 10 % of
     // the best measured plan on every one of them). Time in microseconds of a plan =
     //   rounds * (K blocks per workgroup * c + f)           one workgroup per tile and K split
@@ -244,7 +297,7 @@ int launch(const void *a, const void *b, const float *as, const float *bs, void 
             return fail(RF_ERR_BAD_CONFIG, "unknown schedule");
         }
     } else {
-        select_config(m, n, k, s.num_cu, tiled_ok, &cfg);
+        select_config(m, n, k, s.num_cu, tiled_ok, s.user_plans, &cfg);
     }
 
     if (cfg.variant < 0) {
@@ -349,8 +402,26 @@ int rf_gemm_select_config(int m, int n, int k, rf_gemm_config *out) {
     std::lock_guard<std::mutex> lock(s.mu);
     int rc = ensure_device_info(s);
     if (rc != RF_OK) return rc;
-    select_config(m, n, k, s.num_cu, m >= 16 && n >= 16 && m % 16 == 0 && n % 16 == 0, out);
+    select_config(m, n, k, s.num_cu, m >= 16 && n >= 16 && m % 16 == 0 && n % 16 == 0, s.user_plans, out);
     return RF_OK;
+}
+
+int rf_gemm_load_plans(const char *path, int *count) {
+    g_last_error.clear();
+    if (!path) return fail(RF_ERR_NULL_POINTER, "path is null");
+    State &s = state();
+    std::lock_guard<std::mutex> lock(s.mu);
+    const size_t before = s.user_plans.size();
+    int rc = parse_plans(path, s.user_plans);
+    if (rc != RF_OK) return rc;
+    if (count) *count = (int)(s.user_plans.size() - before);
+    return RF_OK;
+}
+
+void rf_gemm_clear_plans(void) {
+    State &s = state();
+    std::lock_guard<std::mutex> lock(s.mu);
+    s.user_plans.clear();
 }
 
 int rf_gemm_num_variants(void) { return kNumVariants; }

@@ -40,7 +40,7 @@ class PerfMetrics(ctypes.Structure):
 EXPORTS = ("run", "rf_fp8_gemm", "rf_fp8_gemm_ex", "rf_gemm_select_config", "rf_gemm_num_variants",
            "rf_gemm_variant_info", "rf_gemm_variant_has_stream_k", "rf_gemm_variant_has_persistent", "rf_gemm_workspace_bytes", "rf_gemm_init", "rf_gemm_destroy",
            "rf_gemm_last_error", "rf_fp8_gemm_grouped", "rf_quantize_a_f32", "rf_quantize_a_bf16", "rf_quantize_b_f32", "rf_quantize_b_bf16",
-           "rf_cast_f32_to_e4m3fn")
+           "rf_cast_f32_to_e4m3fn", "rf_gemm_load_plans", "rf_gemm_clear_plans")
 
 
 def lib():
@@ -60,6 +60,9 @@ def lib():
         L.rf_fp8_gemm_ex.restype = i32
         L.rf_gemm_select_config.argtypes = [i32, i32, i32, ctypes.POINTER(GemmConfig)]
         L.rf_gemm_select_config.restype = i32
+        L.rf_gemm_load_plans.argtypes = [ctypes.c_char_p, ctypes.POINTER(i32)]
+        L.rf_gemm_load_plans.restype = i32
+        L.rf_gemm_clear_plans.restype = None
         L.rf_gemm_num_variants.restype = i32
         L.rf_gemm_variant_info.argtypes = [i32] + [ctypes.POINTER(i32)] * 5
         L.rf_gemm_variant_info.restype = i32
@@ -217,6 +220,20 @@ def select_config(m, n, k):
     if rc != RF_OK:
         raise RuntimeError("rf_gemm_select_config failed (%d): %s" % (rc, last_error()))
     return cfg
+
+
+def load_plans(path):
+    """Adds the measured plans of a file ("M N K variant split_k group_m stream_k" per line, as written by the tuner's
+    --emit-file) in front of the built-in table; returns how many were added."""
+    n = ctypes.c_int(0)
+    rc = lib().rf_gemm_load_plans(os.fsencode(path), ctypes.byref(n))
+    if rc != RF_OK:
+        raise RuntimeError("rf_gemm_load_plans failed (%d): %s" % (rc, last_error()))
+    return n.value
+
+
+def clear_plans():
+    lib().rf_gemm_clear_plans()
 
 
 def variants():

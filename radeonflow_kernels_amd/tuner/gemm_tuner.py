@@ -8,6 +8,9 @@ DISPATCH_GEMM(...) line. Here nothing is recompiled: every kernel variant is alr
   python -m radeonflow_kernels_amd.tuner.gemm_tuner --M 6144 --N 4608 --K 7168        one shape
   python -m radeonflow_kernels_amd.tuner.gemm_tuner --all --emit                       every known shape, then
                                                                                        rewrite csrc/tuned_plans.inc
+  python -m radeonflow_kernels_amd.tuner.gemm_tuner --M .. --N .. --K .. --emit-file my.plans
+                                                  append the winner to a plan file: rf_gemm_load_plans(path) or the
+                                                  environment variable RF_GEMM_PLANS uses it without a rebuild
 Results go to stdout and, with --out DIR, to DIR/gemm_<M>x<N>x<K>.json (all candidates, best first).
 """
 import argparse
@@ -118,6 +121,7 @@ def main():
     ap.add_argument("--K", type=int)
     ap.add_argument("--all", action="store_true")
     ap.add_argument("--emit", action="store_true", help="rewrite csrc/tuned_plans.inc (rebuild libgemm.so afterwards)")
+    ap.add_argument("--emit-file", default=None, help="append the best plan of every tuned shape to this plan file")
     ap.add_argument("--out", default=None)
     a = ap.parse_args()
     sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
@@ -142,6 +146,14 @@ def main():
     if a.emit:
         emit_plans(results)
         print("wrote", PLANS_INC)
+    if a.emit_file:
+        with open(a.emit_file, "a") as f:
+            for (m, n, k), cands in results.items():
+                if cands:
+                    b = cands[0]
+                    f.write("%d %d %d %d %d %d %d   # %.2f us, %.1f TFLOP/s\n" % (
+                        m, n, k, b["variant"], b["split_k"], b["group_m"], b["stream_k"], b["us"], b["tflops"]))
+        print("appended to", a.emit_file)
 
 
 if __name__ == "__main__":

@@ -42,7 +42,8 @@ def test_python_binding_declares_as_many_arguments_as_the_header():
     from radeonflow_kernels_amd import gemm
     L = gemm.lib()
     counts = _declared_parameter_counts()
-    with_pointers = [n for n in counts if n not in ("rf_gemm_num_variants", "rf_gemm_destroy", "rf_gemm_last_error")]
+    with_pointers = [n for n in counts if n not in ("rf_gemm_num_variants", "rf_gemm_destroy", "rf_gemm_last_error",
+                                                    "rf_gemm_clear_plans")]
     for name in with_pointers:
         at = getattr(L, name).argtypes
         assert at is not None, "%s has no ctypes prototype" % name
@@ -98,3 +99,35 @@ def test_python_mirror_rejects_cpu_tensors_and_wrong_layouts():
     a = torch.zeros((16, 128), dtype=torch.uint8).view(torch.float8_e4m3fn)
     with pytest.raises(ValueError):
         rfk.fp8_mm(a, a, torch.zeros(16, 1), torch.zeros(1, 1), torch.zeros((16, 16), dtype=torch.bfloat16))
+
+
+def test_plan_files_parse_without_a_device(tmp_path):
+    """rf_gemm_load_plans only reads and validates the file (plans are matched against shapes at launch): the tuner's
+    line format, the brace format of csrc/tuned_plans.inc, comments; a bad line fails the whole file and names it."""
+    from radeonflow_kernels_amd import gemm
+    L = gemm.lib()
+    good = tmp_path / "plans.txt"
+    good.write_text("# shape            variant split group schedule\n"
+                    "6144 4608 7168 0 1 16 2\n"
+                    "{1024, 1536, 7168, 3, 4, 8, 0},   // 24.2 us\n"
+                    "\n"
+                    "  512 512 256 1 2 4 0   # trailing comment\n")
+    try:
+        assert gemm.load_plans(str(good)) == 3
+        inc = os.path.join(ROOT, "radeonflow_kernels_amd", "csrc", "tuned_plans.inc")
+        assert gemm.load_plans(inc) == sum(1 for l in open(inc) if l.startswith("{"))
+        n = ctypes.c_int(-1)
+        for text, line in (("512 512 256 1 2 4\n", 1),                       # six fields
+                           ("512 512 256 1 2 4 0\n512 512 200 1 1 4 0\n", 2),   # K not a multiple of 128
+                           ("512 512 256 99 1 4 0\n", 1),                    # no such variant
+                           ("512 512 256 0 2 4 2\n", 1),                     # persistent schedule with a K split
+                           ("512 512 256 0 1 4 0 7\n", 1)):                  # eight fields
+            bad = tmp_path / "bad.txt"
+            bad.write_text(text)
+            assert L.rf_gemm_load_plans(str(bad).encode(), ctypes.byref(n)) == 4
+            assert ("bad.txt:%d" % line).encode() in L.rf_gemm_last_error()
+            assert n.value == -1
+        assert L.rf_gemm_load_plans(str(tmp_path / "missing.txt").encode(), None) == 4
+        assert L.rf_gemm_load_plans(None, None) == 2
+    finally:
+        gemm.clear_plans()

@@ -11,6 +11,7 @@ from helpers import (ATOL, ATOL_REFERENCE, CONFIGS, RTOL, assert_close_to_oracle
                      bf16_bits, exact_problem, oracle_bf16, to_gpu)
 
 pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 @pytest.fixture(scope="module")
@@ -248,3 +249,41 @@ def test_status_codes(rfk):
     bad = rfk.GemmConfig(99, 1, 1, 0)
     assert L.rf_fp8_gemm_ex(p, p, p, p, p, 16, 16, 128, ctypes.byref(bad), None) == 4
     assert b"unsupported shape" in L.rf_gemm_last_error() or L.rf_gemm_last_error() != b""
+
+
+def test_plans_loaded_from_a_file_take_precedence_and_can_be_cleared(rfk, tmp_path):
+    """A plan file changes what the automatic path launches for its shapes (and only for them); results stay bit-exact;
+    a plan that cannot run for its shape is skipped; clearing restores the built-in choice. The environment variable
+    form is checked in a fresh process."""
+    import subprocess
+    import sys
+    m, n, k = 512, 768, 512
+    before = rfk.select_config(m, n, k)
+    other = rfk.select_config(1024, 1536, 7168)
+    forced = (1, 2, 4, 0) if (before.variant, before.split_k) != (1, 2) else (3, 1, 4, 0)
+    path = tmp_path / "my.plans"
+    path.write_text("%d %d %d 0 1 8 2\n" % (m + 16, n, k)                       # persistent on a ragged shape: skipped
+                    + "%d %d %d %d %d %d %d\n" % ((m, n, k) + forced))
+    try:
+        assert rfk.load_plans(str(path)) == 2
+        got = rfk.select_config(m, n, k)
+        assert (got.variant, got.split_k, got.group_m, got.stream_k) == forced
+        ragged = rfk.select_config(m + 16, n, k)
+        assert ragged.stream_k != 2
+        again = rfk.select_config(1024, 1536, 7168)
+        assert (again.variant, again.split_k, again.stream_k) == (other.variant, other.split_k, other.stream_k)
+        data = exact_problem(m, n, k, seed=77)
+        assert np.array_equal(bf16_bits(_run(rfk, data, canary=256)), oracle_bf16(data))
+    finally:
+        rfk.clear_plans()
+    after = rfk.select_config(m, n, k)
+    assert (after.variant, after.split_k, after.stream_k) == (before.variant, before.split_k, before.stream_k)
+    code = ("import radeonflow_kernels_amd as r; c = r.select_config(%d, %d, %d); "
+            "print(c.variant, c.split_k, c.group_m, c.stream_k)" % (m, n, k))
+    env = dict(os.environ, RF_GEMM_PLANS=str(path))
+    out = subprocess.run([sys.executable, "-c", code], env=env, cwd=ROOT, stdout=subprocess.PIPE, text=True, timeout=300)
+    assert out.returncode == 0 and tuple(int(x) for x in out.stdout.split()) == forced
+    env["RF_GEMM_PLANS"] = str(tmp_path / "missing.plans")
+    out = subprocess.run([sys.executable, "-c", code], env=env, cwd=ROOT, stdout=subprocess.PIPE,
+                         stderr=subprocess.PIPE, text=True, timeout=300)
+    assert out.returncode != 0 and "cannot open plan file" in out.stderr
