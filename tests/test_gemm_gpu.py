@@ -287,3 +287,27 @@ def test_plans_loaded_from_a_file_take_precedence_and_can_be_cleared(rfk, tmp_pa
     out = subprocess.run([sys.executable, "-c", code], env=env, cwd=ROOT, stdout=subprocess.PIPE,
                          stderr=subprocess.PIPE, text=True, timeout=300)
     assert out.returncode != 0 and "cannot open plan file" in out.stderr
+
+
+def _random_shapes(count, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        # tile multiples, multiples of 192, ragged multiples of 16 and the occasional odd size, K from 1 to 20 blocks
+        m = int(rng.choice([rng.integers(1, 33) * 128, rng.integers(1, 22) * 192, rng.integers(1, 200) * 16,
+                            rng.integers(1, 700)]))
+        n = int(rng.choice([rng.integers(1, 33) * 128, rng.integers(1, 22) * 192, rng.integers(1, 200) * 16,
+                            rng.integers(1, 700)]))
+        k = int(rng.integers(1, 21)) * 128
+        out.append((m, n, k))
+    return out
+
+
+@pytest.mark.parametrize("m,n,k", _random_shapes(28, seed=20240607))
+def test_automatic_plan_on_random_shapes_is_bit_exact(rfk, m, n, k):
+    """Whatever plan the table or the cost model picks for a shape nobody tuned (any tile family, K split, persistent
+    schedule, bounds-checked kernel), the result on exactly representable data equals the oracle bit for bit and
+    nothing is stored past the end of C."""
+    data = exact_problem(m, n, k, seed=m * 31 + n * 7 + k)
+    out = _run(rfk, data, canary=512)
+    assert np.array_equal(bf16_bits(out), oracle_bf16(data)), "plan %r" % (rfk.select_config(m, n, k),)
