@@ -56,7 +56,8 @@ def _check_canary(buf, used):
 
 CASES = [([256, 128, 512, 64], 512, 256), ([16, 0, 48, 400, 0, 32], 576, 384), ([1024], 256, 512),
          ([128] * 32, 2048, 256), ([0, 0, 272], 144, 128), ([640, 16, 16, 2048, 112], 7168, 256),
-         ([272, 384, 128, 400, 16, 656], 512, 256)]      # left-overs of 16, 128, 128, 144, 16 and 144 rows
+         ([272, 384, 128, 400, 16, 656], 512, 256),      # left-overs of 16, 128, 128, 144, 16 and 144 rows
+         ([int(x) * 16 for x in np.random.default_rng(7).integers(0, 40, 24)], 768, 384)]   # 24 groups of 0..624 rows
 
 
 @pytest.mark.parametrize("rows,n,k", CASES)
