@@ -222,9 +222,10 @@ __global__ __launch_bounds__(256) void quantize_block128(const void *__restrict_
     // ulp of 1 / scale), x * (r * (1 + 2^-20)) and x * (r * (1 - 2^-20)) are, in magnitude, above and below the exact
     // quotient and its fp32 rounding (the factors' rounding errors and the reciprocal's error are below 2^-21
     // together). The fp8 conversion is monotonic, so if the two products convert to the same code, fl32(x / scale)
-    // converts to that code too. Only when they differ (a rounding boundary is that close: about 1 element in 10^5),
-    // or the row contains a NaN, or the scale is so far from 1 that its reciprocal is not a normal number, the group of
-    // four is redone with the division.
+    // converts to that code too. When they differ (a rounding boundary is that close: about 1 element in 10^5 for
+    // fp32 sources, far more often for bf16 ones) the group of four is redone with the exact quotient; when a row
+    // contains a NaN or an infinity, or its scale lies outside (2^-60, 2^60), with the IEEE division and the
+    // NaN-aware encoder.
     float rup[RPT], rdown[RPT];
     bool fast[RPT / 4];
 #pragma unroll
@@ -238,7 +239,7 @@ __global__ __launch_bounds__(256) void quantize_block128(const void *__restrict_
         fast[g] = true;
 #pragma unroll
         for (int j = 0; j < 4; j++)
-            fast[g] = fast[g] && s[4 * g + j] > 0x1p-100f && s[4 * g + j] < 0x1p100f && !has_nan[4 * g + j];
+            fast[g] = fast[g] && s[4 * g + j] > 0x1p-60f && s[4 * g + j] < 0x1p60f && !has_nan[4 * g + j];
     }
 #pragma unroll
     for (int g = 0; g < NG; g++)
@@ -257,9 +258,28 @@ __global__ __launch_bounds__(256) void quantize_block128(const void *__restrict_
             int lo = __builtin_amdgcn_cvt_pk_fp8_f32(yd[0], yd[1], __builtin_bit_cast(int, yd[0]), false);
             lo = __builtin_amdgcn_cvt_pk_fp8_f32(yd[2], yd[3], lo, true);
             uint32_t w = (uint32_t)hi;
-            if (!fast[g] || hi != lo)
+            if (__builtin_expect(!fast[g], 0)) {
                 w = f32x4_to_e4m3fn_codes(v[4 * g][e] / s[4 * g], v[4 * g + 1][e] / s[4 * g + 1],
                                           v[4 * g + 2][e] / s[4 * g + 2], v[4 * g + 3][e] / s[4 * g + 3]);
+            } else if (__builtin_expect(hi != lo, 0)) {
+                // A rounding boundary lies inside the bracket. With bf16 sources that is common, not rare: x and amax
+                // have 8-bit mantissas, so x / scale often IS a boundary (a tie) and one lane in 64 is enough to send
+                // the wave here. The exact quotient decides: the refinement steps of the f32 division expansion
+                // without its range scaling, which the limits on the scale make unnecessary (identical to the IEEE
+                // quotient on 2.9e9 CPU cases, ties of bf16-like operands and reciprocals off by an ulp included).
+                float q[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const float x = v[4 * g + j][e], d = s[4 * g + j];
+                    float r = __builtin_amdgcn_rcpf(d);
+                    r = __builtin_fmaf(__builtin_fmaf(-d, r, 1.0f), r, r);
+                    float t = x * r;
+                    t = __builtin_fmaf(__builtin_fmaf(-d, t, x), r, t);
+                    q[j] = __builtin_copysignf(__builtin_fmaf(__builtin_fmaf(-d, t, x), r, t), x);   // -0 / d stays -0
+                }
+                int c = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], __builtin_bit_cast(int, q[0]), false);
+                w = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], c, true);
+            }
             *(uint32_t *)(tile + (KPT * lane_k + e) * PITCH + row_of(4 * g)) = w;
         }
     __syncthreads();

@@ -39,6 +39,23 @@ def _source(rows, k, seed, kind):
         x *= rng.choice(np.array([-1.0, 1.0], np.float32), x.shape)
         x[:, :, 0] = amax[:, :, 0]                                             # pin the block maximum
         x = x.reshape(rows, k)
+    if kind == "ties":          # bf16-representable sources whose quotients are exact ties or one bf16 step away
+        rng = np.random.default_rng(seed)
+        e = rng.integers(-12, 12, (rows, k // 128, 1))
+        amax = (np.float32(448.0) * np.exp2(e)).astype(np.float32)                # scale = 2^e exactly
+        vals = cref.e4m3fn_to_f32(np.arange(0, 127, dtype=np.uint8))
+        mids = ((vals[:-1] + vals[1:]) / 2).astype(np.float32)                   # at most 5 significant bits
+        x = (mids[rng.integers(0, len(mids), (rows, k // 128, 128))] * np.exp2(e)).astype(np.float32)
+        step = rng.integers(-1, 2, x.shape).astype(np.int32) << 16               # -1, 0, +1 bf16 steps
+        x = (x.view(np.int32) + step).view(np.float32)
+        x *= rng.choice(np.array([-1.0, 1.0], np.float32), x.shape)
+        x[:, :, 0] = amax[:, :, 0]
+        # every fourth block: a maximum with a full bf16 mantissa, so that the scale is not a power of two and the
+        # quotients of small-mantissa values land on and around boundaries by themselves
+        odd = (np.float32(1.0) + rng.integers(1, 128, (rows, k // 128)).astype(np.float32) / np.float32(128.0))
+        x[:, ::4, 0] = (x[:, ::4, 0] * odd[:, ::4] / np.float32(1.75)).astype(np.float32)
+        x = x.reshape(rows, k)
+        x = (x.view(np.uint32) & np.uint32(0xFFFF0000)).view(np.float32)          # bf16-exact
     if kind == "special":       # NaNs of both signs (quiet and signalling patterns), infinities, an all-NaN block
         u = x.view(np.uint32)
         u[0, 5] = 0x7FC00000
@@ -70,7 +87,7 @@ def _unpack(q, s):
     return q.T.contiguous().view(torch.uint8).cpu().numpy(), s.T.contiguous().cpu().numpy()
 
 
-@pytest.mark.parametrize("kind", ["normal", "wide", "boundary", "special"])
+@pytest.mark.parametrize("kind", ["normal", "wide", "boundary", "special", "ties"])
 @pytest.mark.parametrize("rows,k", [(128, 128), (256, 512), (1024, 7168), (576, 1024), (200, 256), (1, 128), (33, 384),
                                     (6144, 256)])
 def test_quantize_a_matches_oracle_bit_for_bit(rfk, rows, k, kind):
@@ -84,7 +101,7 @@ def test_quantize_a_matches_oracle_bit_for_bit(rfk, rows, k, kind):
     assert _codes_equal(a_gpu, a_ref, x)
 
 
-@pytest.mark.parametrize("kind", ["normal", "wide", "boundary", "special"])
+@pytest.mark.parametrize("kind", ["normal", "wide", "boundary", "special", "ties"])
 @pytest.mark.parametrize("rows,k", [(128, 128), (256, 512), (1536, 7168), (576, 1024), (200, 256), (1, 128), (33, 384)])
 def test_quantize_b_matches_oracle_bit_for_bit(rfk, rows, k, kind):
     w = _source(rows, k, 2000 + rows + k, kind)
@@ -97,7 +114,7 @@ def test_quantize_b_matches_oracle_bit_for_bit(rfk, rows, k, kind):
     assert _codes_equal(b_gpu, b_ref, w)
 
 
-@pytest.mark.parametrize("kind", ["normal", "wide", "special"])
+@pytest.mark.parametrize("kind", ["normal", "wide", "special", "ties"])
 @pytest.mark.parametrize("rows,k", [(256, 512), (200, 256)])
 def test_bf16_sources_equal_fp32_sources_of_the_same_values(rfk, rows, k, kind):
     x = torch.from_numpy(_source(rows, k, 77, kind)).bfloat16()
