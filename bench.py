@@ -116,8 +116,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity gate")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build runs on one GPU; --gpus %d is not supported (the path shards over M or N "
-              "without any exchange, see DESIGN.md)" % args.gpus, file=sys.stderr)
+        print("bench.py: this build runs on one GPU; --gpus %d is not supported (output tiles are independent: "
+              "several GPUs would each take a range of rows or columns, with no exchange)" % args.gpus, file=sys.stderr)
         return 2
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
