@@ -33,7 +33,7 @@ SHAPES = [
     (64, 64, 128), (64, 1536, 7168), (64, 3072, 1536), (64, 576, 7168), (96, 7168, 256), (96, 7168, 2048),
     (96, 4608, 7168), (128, 7168, 2304), (128, 512, 7168), (512, 4096, 512), (512, 1536, 7168),
 ]
-SPLITS = (1, 2, 3, 4, 6, 8, 12, 16)
+SPLITS = (1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 16)
 GROUPS = (4, 8, 16)
 
 
