@@ -311,3 +311,39 @@ def test_automatic_plan_on_random_shapes_is_bit_exact(rfk, m, n, k):
     data = exact_problem(m, n, k, seed=m * 31 + n * 7 + k)
     out = _run(rfk, data, canary=512)
     assert np.array_equal(bf16_bits(out), oracle_bf16(data)), "plan %r" % (rfk.select_config(m, n, k),)
+
+
+@pytest.mark.parametrize("m,n,k", [(100, 4096, 512), (1000, 576, 1024), (257, 1000, 256), (1, 4096, 7168), (7, 2050, 384),
+                                   (4097, 130, 256)])
+def test_ragged_shapes_above_the_size_threshold_run_padded_and_bit_exact(rfk, m, n, k):
+    """M or N not a multiple of 16 (or below 16): the operands are staged with padded rows, the tiled kernels run on
+    the padded shape, C comes back without the padding. Exact data must match the oracle bit for bit, nothing may be
+    stored past the end of C, and the reported plan is a tiled one."""
+    assert rfk.select_config(m, n, k).variant >= 0
+    data = exact_problem(m, n, k, seed=3 * m + 5 * n + k)
+    for rep in range(2):                                           # the staging buffer is reused
+        out = _run(rfk, data, canary=777)
+        assert np.array_equal(bf16_bits(out), oracle_bf16(data)), "repetition %d" % rep
+
+
+def test_unaligned_operands_run_padded_and_bit_exact(rfk):
+    """Operands that start 1, 2 and 4 bytes off a 16-byte boundary (views into larger buffers)."""
+    m, n, k = 256, 384, 512
+    data = exact_problem(m, n, k, seed=99)
+    a, b, sa, sb, _ = data
+    dev, fp8 = torch.device("cuda:0"), torch.float8_e4m3fn
+
+    def shifted(t_km, off):                                       # [rows, K] view, stride (1, rows), storage offset off
+        rows = t_km.shape[0]
+        flat = torch.zeros(t_km.numel() + 64, dtype=torch.uint8, device=dev)
+        flat[off:off + t_km.numel()] = t_km.T.contiguous().view(torch.uint8).reshape(-1).to(dev)
+        return flat[off:off + t_km.numel()].view(fp8).view(t_km.shape[1], rows).T
+
+    g = to_gpu(data)
+    cbuf = torch.full((m * n + 64,), -7.0, dtype=torch.bfloat16, device=dev)
+    c = cbuf[2:2 + m * n].view(m, n)                              # 4 bytes off
+    assert c.data_ptr() % 16 == 4
+    rfk.fp8_mm(shifted(a, 1), shifted(b, 2), g[2], g[3], c)
+    torch.cuda.synchronize()
+    assert np.array_equal(bf16_bits(c), oracle_bf16(data))
+    assert float(cbuf[:2].float().abs().max()) == 7.0 and float(cbuf[2 + m * n:].float().abs().min()) == 7.0
