@@ -76,6 +76,13 @@ int rf_fp8_gemm(const void *a, const void *b, const float *as, const float *bs, 
 int rf_fp8_gemm_ex(const void *a, const void *b, const float *as, const float *bs, void *c,
                    int m, int n, int k, const rf_gemm_config *cfg, hipStream_t stream);
 
+/* The same launch `iters` times back to back on `stream`, after `warmup` untimed launches, bracketed by one pair of
+ * events: *us_per_launch receives the average microseconds per launch. For the tuner (the reference's counterpart times
+ * each generated binary with its KernelTimer, tuner/template/gemm_perf.cpp): a host language that needs several
+ * microseconds per call cannot time launches shorter than that from outside. Blocks until the last launch is done. */
+int rf_fp8_gemm_time(const void *a, const void *b, const float *as, const float *bs, void *c, int m, int n, int k,
+                     const rf_gemm_config *cfg, int warmup, int iters, float *us_per_launch, hipStream_t stream);
+
 /* The plan rf_fp8_gemm would use for (m,n,k) on the current device: the gfx950 replacement of the
  * per-shape table in src/gemm/gemm_launcher.cpp:229-259 / tuner/gemm_tuner.py. */
 int rf_gemm_select_config(int m, int n, int k, rf_gemm_config *out);

@@ -484,6 +484,34 @@ int rf_fp8_gemm_ex(const void *a, const void *b, const float *as, const float *b
     return launch(a, b, as, bs, c, m, n, k, cfg, stream);
 }
 
+int rf_fp8_gemm_time(const void *a, const void *b, const float *as, const float *bs, void *c, int m, int n, int k,
+                     const rf_gemm_config *cfg, int warmup, int iters, float *us_per_launch, hipStream_t stream) {
+    if (!us_per_launch || iters < 1 || warmup < 0) {
+        g_last_error.clear();
+        return fail(RF_ERR_BAD_CONFIG, "rf_fp8_gemm_time needs iters >= 1, warmup >= 0 and a result pointer");
+    }
+    for (int i = 0; i < warmup; i++) {
+        int rc = launch(a, b, as, bs, c, m, n, k, cfg, stream);
+        if (rc != RF_OK) return rc;
+    }
+    hipEvent_t e0, e1;
+    RF_HIP(hipEventCreate(&e0));
+    RF_HIP(hipEventCreate(&e1));
+    int rc = RF_OK;
+    hipError_t err = hipEventRecord(e0, stream);
+    for (int i = 0; i < iters && rc == RF_OK && err == hipSuccess; i++) rc = launch(a, b, as, bs, c, m, n, k, cfg, stream);
+    if (err == hipSuccess) err = hipEventRecord(e1, stream);
+    if (err == hipSuccess) err = hipEventSynchronize(e1);
+    float ms = 0.f;
+    if (err == hipSuccess) err = hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (rc != RF_OK) return rc;
+    if (err != hipSuccess) return fail(RF_ERR_HIP, std::string("rf_fp8_gemm_time: ") + hipGetErrorString(err));
+    *us_per_launch = ms * 1e3f / iters;
+    return RF_OK;
+}
+
 int rf_gemm_select_config(int m, int n, int k, rf_gemm_config *out) {
     g_last_error.clear();
     if (!out) return fail(RF_ERR_NULL_POINTER, "out is null");

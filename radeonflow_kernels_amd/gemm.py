@@ -40,7 +40,7 @@ class PerfMetrics(ctypes.Structure):
 EXPORTS = ("run", "rf_fp8_gemm", "rf_fp8_gemm_ex", "rf_gemm_select_config", "rf_gemm_num_variants",
            "rf_gemm_variant_info", "rf_gemm_variant_has_stream_k", "rf_gemm_variant_has_persistent", "rf_gemm_workspace_bytes", "rf_gemm_init", "rf_gemm_destroy",
            "rf_gemm_last_error", "rf_fp8_gemm_grouped", "rf_quantize_a_f32", "rf_quantize_a_bf16", "rf_quantize_b_f32", "rf_quantize_b_bf16",
-           "rf_cast_f32_to_e4m3fn", "rf_gemm_load_plans", "rf_gemm_clear_plans")
+           "rf_cast_f32_to_e4m3fn", "rf_gemm_load_plans", "rf_gemm_clear_plans", "rf_fp8_gemm_time")
 
 
 def lib():
@@ -58,6 +58,9 @@ def lib():
         L.rf_fp8_gemm.restype = i32
         L.rf_fp8_gemm_ex.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, ctypes.POINTER(GemmConfig), vp]
         L.rf_fp8_gemm_ex.restype = i32
+        L.rf_fp8_gemm_time.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, ctypes.POINTER(GemmConfig), i32, i32,
+                                       ctypes.POINTER(ctypes.c_float), vp]
+        L.rf_fp8_gemm_time.restype = i32
         L.rf_gemm_select_config.argtypes = [i32, i32, i32, ctypes.POINTER(GemmConfig)]
         L.rf_gemm_select_config.restype = i32
         L.rf_gemm_load_plans.argtypes = [ctypes.c_char_p, ctypes.POINTER(i32)]
@@ -124,6 +127,21 @@ def fp8_mm(a, b, a_scale, b_scale, c, config=None):
                               m, n, k, cfg, stream)
     if rc != RF_OK:
         raise RuntimeError("rf_fp8_gemm failed (%d): %s" % (rc, last_error()))
+
+
+def fp8_mm_time(a, b, a_scale, b_scale, c, config=None, warmup=3, iters=20):
+    """Average microseconds per launch of fp8_mm over `iters` back-to-back launches timed inside the library (no
+    per-launch Python overhead, which exceeds the GPU time of small shapes)."""
+    m, n, k = _check_layout(a, b, a_scale, b_scale, c)
+    stream = ctypes.c_void_p(torch.cuda.current_stream(a.device).cuda_stream)
+    us = ctypes.c_float(0.0)
+    cfg = ctypes.byref(config) if config is not None else None
+    with torch.cuda.device(a.device):
+        rc = lib().rf_fp8_gemm_time(a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(), c.data_ptr(),
+                                    m, n, k, cfg, warmup, iters, ctypes.byref(us), stream)
+    if rc != RF_OK:
+        raise RuntimeError("rf_fp8_gemm_time failed (%d): %s" % (rc, last_error()))
+    return us.value
 
 
 def fp8_mm_grouped(a, b, a_scale, b_scale, c, row_offsets, variant=-1):

@@ -49,16 +49,8 @@ def _inputs(m, n, k):
 
 
 def _time(rfk, args, cfg, iters):
-    for _ in range(3):
-        rfk.fp8_mm(*args, config=cfg)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(iters):
-        rfk.fp8_mm(*args, config=cfg)
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e3 / iters
+    # timed inside the library: a Python call costs more than the GPU time of the small shapes
+    return rfk.fp8_mm_time(*args, config=cfg, warmup=3, iters=iters)
 
 
 def tune_shape(rfk, m, n, k, log=print):

@@ -347,3 +347,20 @@ def test_unaligned_operands_run_padded_and_bit_exact(rfk):
     torch.cuda.synchronize()
     assert np.array_equal(bf16_bits(c), oracle_bf16(data))
     assert float(cbuf[:2].float().abs().max()) == 7.0 and float(cbuf[2 + m * n:].float().abs().min()) == 7.0
+
+
+
+def test_library_side_timing_loop(rfk):
+    """rf_fp8_gemm_time launches the plan warmup + iters times and reports a plausible average; the result buffer holds
+    the GEMM afterwards; bad arguments are refused."""
+    m, n, k = 256, 384, 512
+    data = exact_problem(m, n, k, seed=4)
+    g = to_gpu(data)
+    us = rfk.fp8_mm_time(*g, warmup=2, iters=50)
+    torch.cuda.synchronize()
+    assert 0.5 < us < 200.0
+    assert np.array_equal(bf16_bits(g[4]), oracle_bf16(data))
+    forced = rfk.fp8_mm_time(*g, config=rfk.GemmConfig(1, 2, 4, 0), warmup=1, iters=10)
+    assert 0.5 < forced < 400.0
+    with pytest.raises(RuntimeError):
+        rfk.fp8_mm_time(*g, iters=0)
