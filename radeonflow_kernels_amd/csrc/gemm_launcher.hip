@@ -239,7 +239,7 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
     // smaller ones never won by more than a few percent.
     struct Candidate { int variant; double c, f; };
     const Candidate cands[] = {{0, 1.355, 9.46}, {3, 0.769, 3.61}, {5, 0.95, 6.0}, {6, 0.65, 4.0}};
-    const double f_next = 3.61, reduce_fixed = 6.83, reduce_per_elem = 8.7e-7;
+    const double f_next = 3.0, reduce_fixed = 6.83, reduce_per_elem = 8.7e-7;
     const int splits_tried[] = {1, 2, 3, 4, 6, 8, 12, 16};
     const int qk = k / rf::BK;
     double best_cost = 1e30;
