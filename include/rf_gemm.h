@@ -125,8 +125,11 @@ void rf_gemm_destroy(void);
  *   c   bf16 [M_total][N]
  *   row_offsets  HOST array of groups+1 ints, row_offsets[0] == 0, non-decreasing; group g owns rows
  *                row_offsets[g] .. row_offsets[g+1]-1 (empty groups allowed); read before the call returns.
- * groups <= 256. Offsets that are all multiples of 16 (with N % 16 == 0 and 16-byte aligned a, b, c) take the tiled
- * kernel in one launch; anything else runs the bounds-checked kernel once per group.
+ * groups <= 256. One launch of the tiled kernel when N % 16 == 0 and b, c are 16-byte aligned. Offsets may be any
+ * numbers (token counts per expert are): when one is not a multiple of 16, or a is not 16-byte aligned, a and as are
+ * first copied into the internal staging buffer with every group starting at a multiple of 16 (one pass over a;
+ * c is written in place, rows of neighbouring groups are not touched). Ragged N, unaligned b or c, and problems below
+ * 2^21 multiply-adds run the bounds-checked kernel once per group.
  * variant: -1 = automatic, else an index into {256x256, 128x256, 128x128, 128x64} tiles, or 4 = 256-row tiles with a
  * 128 x 256 tile for a group's last rows when at most 128 are left. */
 int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const float *bs, void *c, const int *row_offsets,

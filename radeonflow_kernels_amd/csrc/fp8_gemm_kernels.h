@@ -751,10 +751,14 @@ __global__ __launch_bounds__(256) void reduce_splitk_bf16(const float *__restric
 // expert (the reference's consumer is LaunchGroupGEMM over first_token_offset, src/moe/moe.cpp:213-248, which runs
 // fp16 hipBLASLt there). One workgroup per (group, tile): the table is small enough to travel as a kernel argument.
 // Requirements checked by the host: every row_start a multiple of 16 (and so M_total), N % 16 == 0, K % 128 == 0.
+// C may pack the groups more tightly than A does: group g writes out_row_start[g+1] - out_row_start[g] rows from row
+// out_row_start[g] of C, any counts, while its A rows start at row_start[g] and are padded to a multiple of 16 (the
+// host stages A that way when the caller's group sizes are not multiples of 16).
 // ---------------------------------------------------------------------------------------------
 constexpr int kMaxGroups = 256;
 struct GroupTable {
-    int row_start[kMaxGroups + 1];      // prefix of rows
+    int row_start[kMaxGroups + 1];      // first row of each group in A and a_scale (multiples of 16)
+    int out_row_start[kMaxGroups + 1];  // first row of each group in C; the differences are the true row counts
     int tile_start[kMaxGroups + 1];     // prefix of workgroups
 };
 template <int BM, int BN, int WAVES_M, int WAVES_N>
@@ -771,6 +775,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_gro
         if (table.tile_start[mid] <= (int)blockIdx.x) lo = mid; else hi = mid;
     }
     const int grp = lo, row0 = table.row_start[grp], rows = table.row_start[grp + 1] - row0;
+    const int out0 = table.out_row_start[grp], out_rows = table.out_row_start[grp + 1] - out0;
     const int local = blockIdx.x - table.tile_start[grp];
     const int tiles_m = (rows + BM - 1) / BM;
     int tile_m, tile_n;
@@ -780,7 +785,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_gro
     f32x4 acc[G::TM][G::TN];
     tile_mainloop<BM, BN, WAVES_M, WAVES_N>(A + row0, B + (size_t)grp * K * N, SA + row0, SB + (size_t)grp * QK * QN,
                                             rows, M_total, N, m0, n0, 0, QK, lds, acc);
-    store_tile_bf16<BM, BN, WAVES_M, WAVES_N>(acc, C + (size_t)row0 * N, rows, N, m0, n0, lds);
+    store_tile_bf16<BM, BN, WAVES_M, WAVES_N>(acc, C + (size_t)out0 * N, out_rows, N, m0, n0, lds);
 }
 
 // The same with two tile heights in one launch: a group's rows are cut into 256-row tiles, and what is left over
@@ -799,6 +804,7 @@ __global__ __launch_bounds__(512) void gemm_fp8_blockscale_grouped_mixed(
         if (table.tile_start[mid] <= (int)blockIdx.x) lo = mid; else hi = mid;
     }
     const int grp = lo, row0 = table.row_start[grp], rows = table.row_start[grp + 1] - row0;
+    const int out0 = table.out_row_start[grp], out_rows = table.out_row_start[grp + 1] - out0;
     const int local = blockIdx.x - table.tile_start[grp];
     const int big_m = rows / 256 + (rows % 256 > 128 ? 1 : 0);       // 256-row tiles of this group
     const int QK = K / BK, QN = (N + 127) / 128;
@@ -810,13 +816,13 @@ __global__ __launch_bounds__(512) void gemm_fp8_blockscale_grouped_mixed(
         const int m0 = tile_m * 256, n0 = tile_n * 256;
         f32x4 acc[TileGeom<256, 256, 2, 4>::TM][TileGeom<256, 256, 2, 4>::TN];
         tile_mainloop<256, 256, 2, 4>(A + row0, Bg, SA + row0, SBg, rows, M_total, N, m0, n0, 0, QK, lds, acc);
-        store_tile_bf16<256, 256, 2, 4>(acc, C + (size_t)row0 * N, rows, N, m0, n0, lds);
+        store_tile_bf16<256, 256, 2, 4>(acc, C + (size_t)out0 * N, out_rows, N, m0, n0, lds);
     } else {
         const int r1 = row0 + big_m * 256, rest = rows - big_m * 256;  // 16..128 rows
         const int n0 = (local - big_m * tiles_n) * 256;
         f32x4 acc[TileGeom<128, 256, 2, 4>::TM][TileGeom<128, 256, 2, 4>::TN];
         tile_mainloop<128, 256, 2, 4>(A + r1, Bg, SA + r1, SBg, rest, M_total, N, 0, n0, 0, QK, lds, acc);
-        store_tile_bf16<128, 256, 2, 4>(acc, C + (size_t)r1 * N, rest, N, 0, n0, lds);
+        store_tile_bf16<128, 256, 2, 4>(acc, C + (size_t)(out0 + big_m * 256) * N, out_rows - big_m * 256, N, 0, n0, lds);
     }
 }
 

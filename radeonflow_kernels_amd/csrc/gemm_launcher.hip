@@ -389,6 +389,44 @@ int ensure_pad(State &s, size_t bytes) {
     return RF_OK;
 }
 
+// The grouped GEMM's staging copy: the caller's [rows][m_total] matrix (A with T = bytes, a_scale with T = float), in
+// which group g owns columns out_row_start[g] .. out_row_start[g+1]-1, is copied to [rows][m_pad] with group g starting
+// at column row_start[g], a multiple of 16; the columns between a group's end and the next start become zero.
+// blockIdx.y is the group, so the table is read with uniform indices; every thread writes aligned 16-byte pieces.
+// Bytes are fetched as the aligned words that hold them and shifted into place: a source piece starts at any byte.
+template <typename T>
+__global__ __launch_bounds__(256) void pad_group_rows(const T *__restrict__ src, int m_total, int m_pad, int rows,
+                                                      T *__restrict__ dst, const rf::GroupTable table) {
+    constexpr int PER = 16 / sizeof(T);
+    const int g = blockIdx.y, start = table.row_start[g], pieces = (table.row_start[g + 1] - start) / PER;
+    const int from = table.out_row_start[g], count = table.out_row_start[g + 1] - from;
+    const long work = (long)pieces * rows;
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < work; i += (long)gridDim.x * 256) {
+        const int r = (int)(i / pieces), col = (int)(i % pieces) * PER;
+        int valid = count - col;                                       // columns of this piece that exist in the source
+        valid = valid < 0 ? 0 : valid > PER ? PER : valid;
+        const T *p = src + (size_t)r * m_total + from + col;
+        uint32_t out[4];
+        if constexpr (sizeof(T) == 4) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) out[e] = e < valid ? ((const uint32_t *)p)[e] : 0u;
+        } else {
+            const int shift = (int)((uintptr_t)p & 3), need = valid ? shift + valid : 0;
+            const uint32_t *q = (const uint32_t *)((const uint8_t *)p - shift);
+            uint32_t w[5];
+#pragma unroll
+            for (int e = 0; e < 5; e++) w[e] = 4 * e < need ? q[e] : 0u;   // only words that hold a wanted byte
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                out[e] = __builtin_amdgcn_alignbyte(w[e + 1], w[e], shift);
+                const int nv = valid - 4 * e;
+                if (nv < 4) out[e] = nv <= 0 ? 0u : out[e] & ((1u << (8 * nv)) - 1u);
+            }
+        }
+        *(uint4 *)(dst + (size_t)r * m_pad + start + col) = make_uint4(out[0], out[1], out[2], out[3]);
+    }
+}
+
 int launch_padded(State &s, const void *a, const void *b, const float *as, const float *bs, void *c, int m, int n, int k,
                   hipStream_t stream) {
     auto pad16 = [](int x) { return x < 16 ? 16 : (x + 15) / 16 * 16; };
@@ -700,10 +738,12 @@ int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const flo
         g_grouped_attrs_set = true;
     }
     const int qk = k / rf::BK, qn = ceil_div(n, 128);
-    bool tiled = n % 16 == 0 && ((uintptr_t)a % 16) == 0 && ((uintptr_t)b % 16) == 0 && ((uintptr_t)c % 16) == 0;
-    for (int g = 0; g <= groups && tiled; g++) tiled = row_offsets[g] % 16 == 0;
-    if (!tiled) {
-        // ragged groups or unaligned operands: the bounds-checked kernel, one launch per non-empty group
+    const bool direct = n % 16 == 0 && ((uintptr_t)b % 16) == 0 && ((uintptr_t)c % 16) == 0;
+    bool stage = ((uintptr_t)a % 16) != 0;
+    for (int g = 0; g <= groups; g++) stage = stage || row_offsets[g] % 16 != 0;
+    if (!direct || (stage && (double)m_total * n * k < kPadThresholdMacs)) {
+        // ragged N, unaligned weights or output, or next to no work: the bounds-checked kernel, one launch per
+        // non-empty group
         for (int g = 0; g < groups; g++) {
             const int r0 = row_offsets[g], rows = row_offsets[g + 1] - r0;
             if (rows == 0) continue;
@@ -714,6 +754,42 @@ int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const flo
             RF_HIP(hipGetLastError());
         }
         return RF_OK;
+    }
+    rf::GroupTable table;
+    int m_rows = m_total;                      // rows of the A matrix the kernel reads
+    if (stage) {
+        // Group sizes that are not multiples of 16 (token counts per expert never are): A and a_scale are copied
+        // into the staging buffer with every group starting at a multiple of 16, the kernel reads those and writes
+        // each group's true rows straight into the caller's C. Costs one pass over A; the bounds-checked kernel
+        // per group would be 10 to 30 times slower than the tiled one.
+        int at = 0;
+        long most = 0;
+        for (int g = 0; g < groups; g++) {
+            table.row_start[g] = at;
+            const int pr = (row_offsets[g + 1] - row_offsets[g] + 15) / 16 * 16;
+            at += pr;
+            most = pr > most ? pr : most;
+        }
+        for (int g = groups; g <= rf::kMaxGroups; g++) table.row_start[g] = at;
+        for (int g = 0; g <= rf::kMaxGroups; g++) table.out_row_start[g] = row_offsets[g < groups ? g : groups];
+        m_rows = at;
+        const size_t a_bytes = ((size_t)k * m_rows + 255) / 256 * 256;
+        rc = ensure_pad(s, a_bytes + (size_t)qk * m_rows * sizeof(float));
+        if (rc != RF_OK) return rc;
+        auto blocks = [&](long chunks_of_largest_group) {
+            const long x = (chunks_of_largest_group + 256 * 8 - 1) / (256 * 8);
+            return dim3((unsigned)(x < 1 ? 1 : x), groups);
+        };
+        hipLaunchKernelGGL(pad_group_rows<uint8_t>, blocks(most / 16 * k), dim3(256), 0, stream, (const uint8_t *)a,
+                           m_total, m_rows, k, s.pad, table);
+        hipLaunchKernelGGL(pad_group_rows<float>, blocks(most / 4 * qk), dim3(256), 0, stream, as, m_total, m_rows, qk,
+                           (float *)(s.pad + a_bytes), table);
+        RF_HIP(hipGetLastError());
+        a = s.pad;
+        as = (const float *)(s.pad + a_bytes);
+    } else {
+        for (int g = 0; g <= rf::kMaxGroups; g++)
+            table.row_start[g] = table.out_row_start[g] = row_offsets[g < groups ? g : groups];
     }
     if (variant < 0) {
         // the largest tile that still gives every CU a workgroup; failing that, the one with the most workgroups
@@ -739,20 +815,15 @@ int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const flo
         }
     }
     const GroupedVariant &v = kGroupedVariants[variant];
-    rf::GroupTable table;
     const int tiles_n = ceil_div(n, v.bn);
     int tiles = 0;
     for (int g = 0; g < groups; g++) {
-        table.row_start[g] = row_offsets[g];
         table.tile_start[g] = tiles;
         tiles += v.tiles_m(row_offsets[g + 1] - row_offsets[g]) * tiles_n;
     }
-    for (int g = groups; g <= rf::kMaxGroups; g++) {
-        table.row_start[g] = m_total;
-        table.tile_start[g] = tiles;
-    }
+    for (int g = groups; g <= rf::kMaxGroups; g++) table.tile_start[g] = tiles;
     hipLaunchKernelGGL(v.kernel, dim3(tiles), dim3(v.threads), v.lds, stream, (const uint8_t *)a, (const uint8_t *)b, as,
-                       bs, (uint16_t *)c, m_total, n, k, groups, tiles_n, 8, table);
+                       bs, (uint16_t *)c, m_rows, n, k, groups, tiles_n, 8, table);
     RF_HIP(hipGetLastError());
     return RF_OK;
 }

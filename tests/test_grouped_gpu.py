@@ -80,13 +80,55 @@ def test_grouped_quantised_data_within_tolerance(rfk, rows, n, k):
     _check_canary(g[5], g[4].numel())
 
 
-@pytest.mark.parametrize("rows,n,k", [([5, 17, 0, 100], 130, 256), ([33, 64], 72, 128)])
-def test_grouped_ragged_groups_take_the_checked_kernel(rfk, rows, n, k):
+@pytest.mark.parametrize("rows,n,k", [([5, 17, 0, 100], 130, 256), ([33, 64], 72, 128), ([7, 9], 64, 128)])
+def test_grouped_ragged_n_or_tiny_problems_take_the_checked_kernel(rfk, rows, n, k):
     g, offs, exp = _grouped_problem(rows, n, k, seed=3, exact=True)
     rfk.fp8_mm_grouped(*g[:5], offs)
     torch.cuda.synchronize()
     assert np.array_equal(bf16_bits(g[4]), exp)
     _check_canary(g[5], g[4].numel())
+
+
+RAGGED = [([5, 17, 0, 100, 333, 1], 512, 256), ([1, 1, 1, 1, 300], 256, 384), ([255, 257, 129, 0, 143, 15], 768, 256),
+          ([1000], 256, 128), ([int(x) for x in np.random.default_rng(3).integers(0, 300, 40)], 576, 256)]
+
+
+@pytest.mark.parametrize("rows,n,k", RAGGED)
+def test_grouped_any_group_sizes_bit_exact(rfk, rows, n, k):
+    """Group sizes that are not multiples of 16 (what token routing produces): A is staged with padded groups, C is
+    written in place, so rows of the next group must survive and nothing may land past the end."""
+    g, offs, exp = _grouped_problem(rows, n, k, seed=31 + n, exact=True)
+    for variant in (-1, 0, 1, 2, 3, 4):
+        g[4].fill_(-3.0)
+        rfk.fp8_mm_grouped(*g[:5], offs, variant=variant)
+        torch.cuda.synchronize()
+        assert np.array_equal(bf16_bits(g[4]), exp), "variant %d" % variant
+        _check_canary(g[5], g[4].numel())
+
+
+def test_grouped_any_group_sizes_quantised_data(rfk):
+    rows, n, k = [77, 130, 1, 260, 45], 1024, 1024
+    g, offs, exp = _grouped_problem(rows, n, k, seed=8, exact=False)
+    rfk.fp8_mm_grouped(*g[:5], offs)
+    torch.cuda.synchronize()
+    assert_close_to_oracle(g[4], exp, RTOL, ATOL, "grouped, ragged sizes")
+    _check_canary(g[5], g[4].numel())
+
+
+@pytest.mark.parametrize("shift", [1, 2, 3, 7])
+def test_grouped_unaligned_a(rfk, shift):
+    """A that does not start on a 16-byte boundary (a view into a larger buffer) goes through the same staging copy."""
+    rows, n, k = [48, 100, 16], 256, 256
+    g, offs, exp = _grouped_problem(rows, n, k, seed=2, exact=True)
+    a = g[0]
+    m_total = a.shape[0]
+    raw = torch.zeros(k * m_total + 64, dtype=torch.uint8, device=a.device)
+    raw[shift:shift + k * m_total] = a.T.contiguous().view(torch.uint8).reshape(-1)
+    a2 = raw[shift:shift + k * m_total].view(k, m_total).view(torch.float8_e4m3fn).T
+    assert a2.data_ptr() % 16 == shift
+    rfk.fp8_mm_grouped(a2, *g[1:5], offs)
+    torch.cuda.synchronize()
+    assert np.array_equal(bf16_bits(g[4]), exp)
 
 
 def test_grouped_equals_separate_gemms(rfk):
