@@ -262,22 +262,26 @@ def main():
         gsa = (torch.rand((gk // 128, gm), device="cuda") * 1e-2).T
         gsb = (torch.rand((gg, gk // 128, gn // 128), device="cuda") * 1e-2).permute(0, 2, 1)
         gc = torch.empty((gm, gn), dtype=torch.bfloat16, device="cuda")
-        with torch.cuda.stream(stream):
-            for _ in range(args.warmup // 4 + 5):
-                rfk.fp8_mm_grouped(ga, gb, gsa, gsb, gc, offs)
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(stream)
-            for _ in range(50):
-                rfk.fp8_mm_grouped(ga, gb, gsa, gsb, gc, offs)
-            e1.record(stream)
-            stream.synchronize()
-        u = e0.elapsed_time(e1) * 1e3 / 50
-        tf = 2.0 * gm * gn * gk / u / 1e6
-        out["grouped"] = {"workload": "32 groups, %d rows in total (16..%d per group), N=%d K=%d" % (
-                              gm, max(b - a for a, b in zip(offs, offs[1:])), gn, gk),
-                          "us": round(u, 2), "tflops": round(tf, 1), "pct_fp8_mfma_peak": round(100 * tf / PEAK_FP8_TFLOPS, 2)}
-        print("grouped %s: %.2f us  %.1f TFLOP/s (%.1f %% of peak)" % (out["grouped"]["workload"], u, tf,
-              100 * tf / PEAK_FP8_TFLOPS), file=sys.stderr)
+        # the same rows cut at arbitrary places (what token routing gives): A is staged with padded groups first
+        cuts_any = np.sort(rng.choice(np.arange(1, 8192), 31, replace=False))
+        for key, offs_ in (("grouped", offs), ("grouped_any_sizes", [0] + [int(x) for x in cuts_any] + [8192])):
+            with torch.cuda.stream(stream):
+                for _ in range(args.warmup // 4 + 5):
+                    rfk.fp8_mm_grouped(ga, gb, gsa, gsb, gc, offs_)
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                for _ in range(50):
+                    rfk.fp8_mm_grouped(ga, gb, gsa, gsb, gc, offs_)
+                e1.record(stream)
+                stream.synchronize()
+            u = e0.elapsed_time(e1) * 1e3 / 50
+            tf = 2.0 * gm * gn * gk / u / 1e6
+            sizes = [b - a for a, b in zip(offs_, offs_[1:])]
+            out[key] = {"workload": "32 groups, %d rows in total (%d..%d per group), N=%d K=%d" % (
+                            gm, min(sizes), max(sizes), gn, gk),
+                        "us": round(u, 2), "tflops": round(tf, 1), "pct_fp8_mfma_peak": round(100 * tf / PEAK_FP8_TFLOPS, 2)}
+            print("%s %s: %.2f us  %.1f TFLOP/s (%.1f %% of peak)" % (key, out[key]["workload"], u, tf,
+                  100 * tf / PEAK_FP8_TFLOPS), file=sys.stderr)
         # the same launch with other operand bits (same shapes, scales and plan): the chip's clock under load depends
         # on how many bits toggle, so the time does too
         out["operand_bits"] = {"quantised_normal_us": round(us, 2)}

@@ -358,22 +358,6 @@ int launch_locked(State &s, const void *a, const void *b, const float *as, const
 // copied into a staging buffer with rows padded to a multiple of 16 (zeros: padded rows and columns produce values
 // nobody reads), the tiled kernels run on the padded shape under the automatic plan, and C is copied back without the
 // padding. b_scale needs no copy: ceil(N/128) does not change. The copies cost K*M (+ K*N when N is ragged) bytes.
-template <typename T>
-__global__ __launch_bounds__(256) void pad_columns(const T *__restrict__ src, int cols, int cols_pad, int rows,
-                                                   T *__restrict__ dst) {
-    constexpr int PER = 16 / sizeof(T);                    // one aligned 16-byte store per thread
-    const size_t chunk = (size_t)blockIdx.x * 256 + threadIdx.x, chunks_per_row = cols_pad / PER;
-    if (chunk >= chunks_per_row * rows) return;
-    const size_t r = chunk / chunks_per_row;
-    const int c0 = (int)(chunk % chunks_per_row) * PER;
-    T v[PER];
-#pragma unroll
-    for (int e = 0; e < PER; e++) v[e] = c0 + e < cols ? src[r * cols + c0 + e] : T(0);
-    T *out = dst + r * cols_pad + c0;
-#pragma unroll
-    for (int e = 0; e < PER; e++) out[e] = v[e];
-}
-
 constexpr double kPadThresholdMacs = 2097152.0;            // below this the bounds-checked kernel is as fast
 
 int ensure_pad(State &s, size_t bytes) {
@@ -427,6 +411,26 @@ __global__ __launch_bounds__(256) void pad_group_rows(const T *__restrict__ src,
     }
 }
 
+// grid of pad_group_rows: enough workgroups for one piece per thread, capped (threads loop over the rest)
+dim3 pad_grid(long pieces_of_largest_group, int groups) {
+    long x = (pieces_of_largest_group + 255) / 256;
+    const long cap = 4096 / groups > 0 ? 4096 / groups : 1;
+    x = x < 1 ? 1 : x > cap ? cap : x;
+    return dim3((unsigned)x, (unsigned)groups);
+}
+
+// table of one group of `cols` columns padded to `cols_pad`
+rf::GroupTable one_group(int cols, int cols_pad) {
+    rf::GroupTable t;
+    t.row_start[0] = t.out_row_start[0] = t.tile_start[0] = 0;
+    for (int g = 1; g <= rf::kMaxGroups; g++) {
+        t.row_start[g] = cols_pad;
+        t.out_row_start[g] = cols;
+        t.tile_start[g] = 0;
+    }
+    return t;
+}
+
 int launch_padded(State &s, const void *a, const void *b, const float *as, const float *bs, void *c, int m, int n, int k,
                   hipStream_t stream) {
     auto pad16 = [](int x) { return x < 16 ? 16 : (x + 15) / 16 * 16; };
@@ -441,23 +445,22 @@ int launch_padded(State &s, const void *a, const void *b, const float *as, const
     const size_t off_c = off;  off += copy_c ? align((size_t)mp * np * 2) : 0;
     int rc = ensure_pad(s, off);
     if (rc != RF_OK) return rc;
-    auto blocks = [](size_t chunks) { return dim3((unsigned)((chunks + 255) / 256)); };
     const void *a2 = a, *b2 = b;
     const float *as2 = as;
     void *c2 = c;
     if (copy_a) {
-        hipLaunchKernelGGL(pad_columns<uint8_t>, blocks((size_t)k * (mp / 16)), dim3(256), 0, stream, (const uint8_t *)a, m,
-                           mp, k, s.pad + off_a);
+        hipLaunchKernelGGL(pad_group_rows<uint8_t>, pad_grid((long)k * (mp / 16), 1), dim3(256), 0, stream,
+                           (const uint8_t *)a, m, mp, k, s.pad + off_a, one_group(m, mp));
         a2 = s.pad + off_a;
     }
     if (copy_b) {
-        hipLaunchKernelGGL(pad_columns<uint8_t>, blocks((size_t)k * (np / 16)), dim3(256), 0, stream, (const uint8_t *)b, n,
-                           np, k, s.pad + off_b);
+        hipLaunchKernelGGL(pad_group_rows<uint8_t>, pad_grid((long)k * (np / 16), 1), dim3(256), 0, stream,
+                           (const uint8_t *)b, n, np, k, s.pad + off_b, one_group(n, np));
         b2 = s.pad + off_b;
     }
     if (copy_sa) {
-        hipLaunchKernelGGL(pad_columns<float>, blocks((size_t)qk * (mp / 4)), dim3(256), 0, stream, as, m, mp, qk,
-                           (float *)(s.pad + off_sa));
+        hipLaunchKernelGGL(pad_group_rows<float>, pad_grid((long)qk * (mp / 4), 1), dim3(256), 0, stream, as, m, mp, qk,
+                           (float *)(s.pad + off_sa), one_group(m, mp));
         as2 = (const float *)(s.pad + off_sa);
     }
     if (copy_c) c2 = s.pad + off_c;
@@ -776,14 +779,10 @@ int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const flo
         const size_t a_bytes = ((size_t)k * m_rows + 255) / 256 * 256;
         rc = ensure_pad(s, a_bytes + (size_t)qk * m_rows * sizeof(float));
         if (rc != RF_OK) return rc;
-        auto blocks = [&](long chunks_of_largest_group) {
-            const long x = (chunks_of_largest_group + 256 * 8 - 1) / (256 * 8);
-            return dim3((unsigned)(x < 1 ? 1 : x), groups);
-        };
-        hipLaunchKernelGGL(pad_group_rows<uint8_t>, blocks(most / 16 * k), dim3(256), 0, stream, (const uint8_t *)a,
-                           m_total, m_rows, k, s.pad, table);
-        hipLaunchKernelGGL(pad_group_rows<float>, blocks(most / 4 * qk), dim3(256), 0, stream, as, m_total, m_rows, qk,
-                           (float *)(s.pad + a_bytes), table);
+        hipLaunchKernelGGL(pad_group_rows<uint8_t>, pad_grid(most / 16 * k, groups), dim3(256), 0, stream,
+                           (const uint8_t *)a, m_total, m_rows, k, s.pad, table);
+        hipLaunchKernelGGL(pad_group_rows<float>, pad_grid(most / 4 * qk, groups), dim3(256), 0, stream, as, m_total,
+                           m_rows, qk, (float *)(s.pad + a_bytes), table);
         RF_HIP(hipGetLastError());
         a = s.pad;
         as = (const float *)(s.pad + a_bytes);
