@@ -70,6 +70,59 @@ def time_gemm(rfk, sets, steps, warmup, stream):
     return e0.elapsed_time(e1) * 1e3 / steps
 
 
+def clock_under_load(rfk, g, seconds, us_per_launch):
+    """Shader clock and board power while the GEMM runs back to back for `seconds`, read from the amdgpu driver's
+    sysfs files (pp_dpm_sclk, hwmon power1_input / power1_average) by a polling thread; the launches are issued by
+    the library's own timing loop, which does not hold the interpreter lock. None where the files cannot be read."""
+    import glob
+    import threading
+    cards = [c for c in sorted(glob.glob("/sys/class/drm/card*/device")) if os.path.exists(c + "/pp_dpm_sclk")]
+    if not cards:
+        return None
+
+    def sample():
+        best = None
+        for card in cards:
+            try:
+                cur = [l for l in open(card + "/pp_dpm_sclk").read().splitlines() if l.rstrip().endswith("*")]
+                mhz = float(cur[0].split(":")[1].lower().replace("mhz", "").replace("*", "").strip())
+                watts = None
+                for f in glob.glob(card + "/hwmon/hwmon*/power1_input") + glob.glob(card + "/hwmon/hwmon*/power1_average"):
+                    watts = float(open(f).read()) / 1e6
+                    break
+            except (OSError, ValueError, IndexError):
+                continue
+            if best is None or mhz > best[0]:
+                best = (mhz, watts)
+        return best
+
+    got, done = [], threading.Event()
+
+    def poll():
+        while not done.is_set():
+            v = sample()
+            if v:
+                got.append(v)
+            time.sleep(0.02)
+
+    t = threading.Thread(target=poll)
+    t.start()
+    try:
+        us = rfk.fp8_mm_time(*g, warmup=20, iters=max(50, int(seconds * 1e6 / us_per_launch)))
+    finally:
+        done.set()
+        t.join()
+    got = got[len(got) // 3:]            # the clock needs tens of milliseconds to settle
+    if not got:
+        return None
+    watts = [w for _, w in got if w is not None]
+    mhz = sum(v for v, _ in got) / len(got)
+    return {"sclk_mhz": round(mhz, 1), "power_w": round(sum(watts) / len(watts), 1) if watts else None,
+            "us_per_gemm": round(us, 2), "samples": len(got),
+            "fp8_peak_at_this_clock_tflops": round(PEAK_FP8_TFLOPS * mhz / 2400.0, 1),
+            "source": "sysfs pp_dpm_sclk and hwmon power, mean over the last two thirds of %.1f s of back-to-back launches" % seconds}
+
+
 def per_launch_us(rfk, g, launches, stream):
     """Each launch bracketed by its own pair of HIP events (clocks already warm): list of microseconds."""
     with torch.cuda.stream(stream):
@@ -187,6 +240,9 @@ def main():
                    "derived_fp8_peak_tflops": round(derived_peak, 1), "input_generation_s": round(gen_s, 2)},
         "roofline": roofline,
     }
+
+    with torch.cuda.stream(stream):
+        out["clock_under_load"] = clock_under_load(rfk, g, 0.6, us)
 
     if not args.no_cpu:
         # CPU baseline = the oracle's torch restatement of the reference path (dequantise, fp32 matmul, bf16)
