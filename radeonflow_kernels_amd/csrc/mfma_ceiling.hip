@@ -1,6 +1,6 @@
 // Measures what the whole gfx950 chip sustains on the fp8 MFMA the GEMM is built on when nothing else runs:
 // 8 waves per compute unit issue v_mfma_f32_16x16x128_f8f6f4 back to back from registers (8 independent
-// accumulators per wave, no memory, no LDS). The published peak (5.0 PFLOP/s dense) assumes 2.4 GHz; under load the
+// accumulators per wave over 4 x 2 operand fragments, no memory, no LDS). The published peak (5.0 PFLOP/s dense) assumes 2.4 GHz; under load the
 // chip lowers its clock to stay inside its power limit, and how far depends on how many bits toggle in the operands.
 // The figure for realistic operands is the ceiling any fp8 GEMM on this chip can approach.
 //
@@ -23,19 +23,23 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 constexpr int kAcc = 8, kWords = 4096;
 
 __global__ __launch_bounds__(512) void mfma_from_registers(const int *__restrict__ src, float *out, int iters) {
-    i32x8 a, b;
+    // 4 x 2 operand fragments, as a wave tile of a GEMM holds them: consecutive MFMAs see different operand bits
+    i32x8 a[4], b[2];
 #pragma unroll
-    for (int e = 0; e < 8; e++) {
-        a[e] = src[(threadIdx.x * 8 + e) % kWords];
-        b[e] = src[(threadIdx.x * 8 + e + kWords / 2) % kWords];
-    }
+    for (int f = 0; f < 4; f++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) a[f][e] = src[(threadIdx.x * 8 + e + f * 517) % kWords];
+#pragma unroll
+    for (int f = 0; f < 2; f++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) b[f][e] = src[(threadIdx.x * 8 + e + kWords / 2 + f * 1031) % kWords];
     f32x4 acc[kAcc];
 #pragma unroll
     for (int r = 0; r < kAcc; r++) acc[r] = (f32x4){0.f, 0.f, 0.f, 0.f};
     for (int it = 0; it < iters; it++) {
 #pragma unroll
         for (int r = 0; r < kAcc; r++)
-            acc[r] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[r], 0, 0, 0, 0, 0, 0);
+            acc[r] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a[r % 4], b[r / 4], acc[r], 0, 0, 0, 0, 0, 0);
     }
     float s = 0.f;
 #pragma unroll
