@@ -106,7 +106,8 @@ int rf_gemm_variant_info(int variant, int *block_m, int *block_n, int *waves_m, 
 int rf_gemm_variant_has_stream_k(int variant);
 int rf_gemm_variant_has_persistent(int variant);
 
-/* Device workspace (split-K partial sums) needed for a shape under the automatic plan, in bytes. */
+/* Device workspace (split-K partial sums) needed for a shape under the automatic plan, in bytes. The staging copies
+ * of ragged or unaligned operands are not part of it: that buffer grows on the first such call. */
 size_t rf_gemm_workspace_bytes(int m, int n, int k);
 
 /* Optional explicit set-up / tear-down of the process-wide workspace on the current device. run() and
