@@ -364,3 +364,46 @@ def test_library_side_timing_loop(rfk):
     assert 0.5 < forced < 400.0
     with pytest.raises(RuntimeError):
         rfk.fp8_mm_time(*g, iters=0)
+
+
+def test_hip_graph_replays_match_eager(rfk):
+    """Quantiser + GEMM (automatic plan, a split-K plan with its reduction, the persistent schedule) captured into one
+    HIP graph: every replay, with new inputs and eager launches in between, gives the bits of the eager run. The
+    library allocates nothing during the capture because the eager runs before it have grown the split-K workspace."""
+    m, n, k = 512, 512, 1024
+    dev = torch.device("cuda:0")
+    gen = torch.Generator().manual_seed(5)
+    b, sb = rfk.quantize_b(torch.randn((n, k), generator=gen).to(dev))
+    xs = [torch.randn((m, k), generator=gen).to(dev) for _ in range(4)]
+    plans = [None, rfk.GemmConfig(3, 4, 8, 0), rfk.GemmConfig(0, 1, 4, 2)]
+
+    def step(x, outs):
+        a, sa = rfk.quantize_a(x)
+        for c, plan in zip(outs, plans):
+            rfk.fp8_mm(a, b, sa, sb, c, config=plan)
+
+    def outputs():
+        return [torch.zeros((m, n), dtype=torch.bfloat16, device=dev) for _ in plans]
+
+    eager = [outputs() for _ in xs]
+    for x, outs in zip(xs, eager):
+        step(x, outs)
+    torch.cuda.synchronize()
+    assert not torch.equal(eager[0][0], eager[1][0])
+    x_static, outs_static = xs[0].clone(), outputs()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(x_static, outs_static)
+    for i in (1, 2, 3, 0, 2):
+        x_static.copy_(xs[i])
+        for c in outs_static:
+            c.fill_(-1.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for c, e, plan in zip(outs_static, eager[i], plans):
+            assert torch.equal(c.view(torch.uint16), e.view(torch.uint16)), "replay with input %d, plan %r" % (i, plan)
+        again = outputs()                      # the program's own eager work between two replays
+        step(xs[(i + 1) % 4], again)
+        torch.cuda.synchronize()
+        assert torch.equal(again[1].view(torch.uint16), eager[(i + 1) % 4][1].view(torch.uint16))
