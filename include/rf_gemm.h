@@ -13,7 +13,7 @@
  * Shapes with M%16==0, N%16==0 and 16-byte aligned a/b/c take the tiled MFMA path as they are. Anything else is
  * staged: the operands that need it are copied with rows padded to a multiple of 16 (zeros) into an internal buffer
  * grown on demand, the tiled path runs on the padded shape, and c receives the result without the padding (cost: one
- * pass over a, plus one over b when N is ragged). Problems below 2^21 multiply-adds, and explicit plans with
+ * pass over a; when N is ragged or c unaligned also one over b and a staged copy of c). Problems below 2^21 multiply-adds, and explicit plans with
  * variant = -1, take a bounds-checked kernel instead (the role of the reference's legacy kernel,
  * src/gemm/gemm_kernel_legacy.cpp:237-374).
  * Not thread-safe across host threads (one lazily grown workspace per process), like the reference.

@@ -635,7 +635,8 @@ __device__ __forceinline__ void exchange_tile_f32(f32x4 (&acc)[BM / WAVES_M / 16
 
 // ---------------------------------------------------------------------------------------------
 // One workgroup per (tile, K split). PARTIAL=false: writes bf16 C. PARTIAL=true: writes the fp32 partial sums of
-// the K range of split blockIdx.y to ws[split][M][N] (summed by reduce_splitk_bf16).
+// the K range of split blockIdx.y to ws[split][M][N] (summed by reduce_splitk_bf16). M_store <= M is the number of
+// rows of bf16 C that exist (a caller whose M is not a multiple of 16 passes A padded to M rows and its own C).
 // Requirements checked by the host: M%16==0, N%16==0, M>=16, N>=16, a/b 16-byte aligned,
 // c 16-byte aligned, K%128==0.
 // ---------------------------------------------------------------------------------------------
@@ -643,7 +644,7 @@ template <int BM, int BN, int WAVES_M, int WAVES_N, bool PARTIAL, int NS = 2>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_tile(
     const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
     const float *__restrict__ SB, void *__restrict__ Cout, int M, int N, int K, int kb_per_split,
-    int tiles_m, int tiles_n, int group_m) {
+    int tiles_m, int tiles_n, int group_m, int M_store) {
     using G = TileGeom<BM, BN, WAVES_M, WAVES_N>;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     int tile_m, tile_n;
@@ -658,7 +659,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
         store_tile_f32_staged<BM, BN, WAVES_M, WAVES_N>(acc, (float *)Cout + ((size_t)blockIdx.y * M + m0) * N + n0, N,
                                                         M - m0, N - n0, lds);
     else
-        store_tile_bf16<BM, BN, WAVES_M, WAVES_N>(acc, (uint16_t *)Cout, M, N, m0, n0, lds);
+        store_tile_bf16<BM, BN, WAVES_M, WAVES_N>(acc, (uint16_t *)Cout, M_store, N, m0, n0, lds);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -729,13 +730,14 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_str
 
 // Sum of split-K partials in split order 0..S-1, then one bf16 rounding
 // (the reference's reduce_kernel, src/gemm/gemm_kernel.cpp:288-303). 4 outputs per thread.
+// mn: elements of C; split_stride: elements between two splits in ws (>= mn: the partials may have more rows than C).
 __global__ __launch_bounds__(256) void reduce_splitk_bf16(const float *__restrict__ ws, uint16_t *__restrict__ C,
-                                                          size_t mn, int splits) {
+                                                          size_t mn, int splits, size_t split_stride) {
     size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= mn) return;
     f32x4 s = *(const f32x4 *)(ws + i);
     for (int p = 1; p < splits; p++) {
-        f32x4 v = *(const f32x4 *)(ws + (size_t)p * mn + i);
+        f32x4 v = *(const f32x4 *)(ws + (size_t)p * split_stride + i);
         s[0] += v[0]; s[1] += v[1]; s[2] += v[2]; s[3] += v[3];
     }
     uint2 o;

@@ -35,7 +35,7 @@ int fail(int code, const std::string &msg) {
 
 // ---- variant table -------------------------------------------------------------------------
 typedef void (*tile_kernel_t)(const uint8_t *, const uint8_t *, const float *, const float *, void *, int, int, int,
-                              int, int, int, int);
+                              int, int, int, int, int);
 typedef void (*streamk_kernel_t)(const uint8_t *, const uint8_t *, const float *, const float *, uint16_t *, int, int,
                                  int, int, int, int, unsigned *, float *);
 typedef void (*persistent_kernel_t)(const uint8_t *, const uint8_t *, const float *, const float *, uint16_t *, int, int,
@@ -266,10 +266,12 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
     }
 }
 
-// The launch proper; the caller holds the lock and has checked shape and pointers.
+// The launch proper; the caller holds the lock and has checked shape and pointers. m_store >= 0: c has only m_store
+// (<= m) rows, the rest of the m rows of the operands are padding (one workgroup per tile schedules only).
 int launch_locked(State &s, const void *a, const void *b, const float *as, const float *bs, void *c, int m, int n, int k,
-                  const rf_gemm_config *user_cfg, hipStream_t stream) {
+                  const rf_gemm_config *user_cfg, hipStream_t stream, int m_store = -1) {
     int rc = RF_OK;
+    if (m_store < 0) m_store = m;
     const bool tiled_ok = tiled_path_ok(a, b, c, m, n);
     rf_gemm_config cfg;
     if (user_cfg) {
@@ -294,6 +296,8 @@ int launch_locked(State &s, const void *a, const void *b, const float *as, const
         select_config(m, n, k, s.num_cu, tiled_ok, s.user_plans, &cfg);
     }
 
+    if (m_store != m && (cfg.variant < 0 || cfg.stream_k != RF_SCHEDULE_TILES))
+        return fail(RF_ERR_BAD_CONFIG, "internal: this schedule cannot write fewer rows than it computes");
     if (cfg.variant < 0) {
         dim3 grid(ceil_div(n, 16), ceil_div(m, 16));
         hipLaunchKernelGGL(rf::gemm_fp8_blockscale_checked, grid, dim3(64), 0, stream, (const uint8_t *)a,
@@ -335,17 +339,18 @@ int launch_locked(State &s, const void *a, const void *b, const float *as, const
     }
     if (splits == 1) {
         hipLaunchKernelGGL(v.direct, grid, block, v.lds_bytes(), stream, (const uint8_t *)a, (const uint8_t *)b, as, bs,
-                           c, m, n, k, kb_per_split, tiles_m, tiles_n, cfg.group_m);
+                           c, m, n, k, kb_per_split, tiles_m, tiles_n, cfg.group_m, m_store);
         RF_HIP(hipGetLastError());
     } else {
         const size_t mn = (size_t)m * n;
         rc = ensure_workspace(s, mn * splits * sizeof(float));
         if (rc != RF_OK) return rc;
         hipLaunchKernelGGL(v.partial, grid, block, v.lds_bytes(), stream, (const uint8_t *)a, (const uint8_t *)b, as,
-                           bs, (void *)s.ws, m, n, k, kb_per_split, tiles_m, tiles_n, cfg.group_m);
+                           bs, (void *)s.ws, m, n, k, kb_per_split, tiles_m, tiles_n, cfg.group_m, m);
         RF_HIP(hipGetLastError());
-        hipLaunchKernelGGL(rf::reduce_splitk_bf16, dim3((unsigned)((mn / 4 + 255) / 256)), dim3(256), 0, stream,
-                           (const float *)s.ws, (uint16_t *)c, mn, splits);
+        const size_t mn_store = (size_t)m_store * n;
+        hipLaunchKernelGGL(rf::reduce_splitk_bf16, dim3((unsigned)((mn_store / 4 + 255) / 256)), dim3(256), 0, stream,
+                           (const float *)s.ws, (uint16_t *)c, mn_store, splits, mn);
         RF_HIP(hipGetLastError());
     }
     return RF_OK;
@@ -437,7 +442,12 @@ int launch_padded(State &s, const void *a, const void *b, const float *as, const
     auto align = [](size_t x) { return (x + 255) / 256 * 256; };
     const int mp = pad16(m), np = pad16(n), qk = k / rf::BK;
     const bool copy_a = mp != m || (uintptr_t)a % 16 != 0, copy_b = np != n || (uintptr_t)b % 16 != 0;
-    const bool copy_sa = mp != m, copy_c = mp != m || np != n || (uintptr_t)c % 16 != 0;
+    const bool copy_sa = mp != m;
+    // The plan of the padded shape. With whole columns and an aligned c, a plan of one workgroup per tile writes the m
+    // true rows straight into c (its stores are masked by row); otherwise C is staged and copied back.
+    rf_gemm_config cfg;
+    select_config(mp, np, k, s.num_cu, true, s.user_plans, &cfg);
+    const bool copy_c = np != n || (uintptr_t)c % 16 != 0 || (mp != m && cfg.stream_k != RF_SCHEDULE_TILES);
     size_t off = 0;
     const size_t off_a = off;  off += copy_a ? align((size_t)k * mp) : 0;
     const size_t off_b = off;  off += copy_b ? align((size_t)k * np) : 0;
@@ -465,7 +475,7 @@ int launch_padded(State &s, const void *a, const void *b, const float *as, const
     }
     if (copy_c) c2 = s.pad + off_c;
     RF_HIP(hipGetLastError());
-    rc = launch_locked(s, a2, b2, as2, bs, c2, mp, np, k, nullptr, stream);
+    rc = launch_locked(s, a2, b2, as2, bs, c2, mp, np, k, &cfg, stream, copy_c ? mp : m);
     if (rc != RF_OK) return rc;
     if (copy_c)
         RF_HIP(hipMemcpy2DAsync(c, (size_t)n * 2, c2, (size_t)np * 2, (size_t)n * 2, m, hipMemcpyDeviceToDevice, stream));

@@ -314,10 +314,11 @@ def test_automatic_plan_on_random_shapes_is_bit_exact(rfk, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(100, 4096, 512), (1000, 576, 1024), (257, 1000, 256), (1, 4096, 7168), (7, 2050, 384),
-                                   (4097, 130, 256)])
+                                   (4097, 130, 256), (1020, 768, 512), (500, 1536, 2048), (2040, 2048, 256)])
 def test_ragged_shapes_above_the_size_threshold_run_padded_and_bit_exact(rfk, m, n, k):
     """M or N not a multiple of 16 (or below 16): the operands are staged with padded rows, the tiled kernels run on
-    the padded shape, C comes back without the padding. Exact data must match the oracle bit for bit, nothing may be
+    the padded shape; C is written in place when only M is ragged (directly or by the split-K reduction) and comes
+    back from a staged copy otherwise (ragged N, or a padded M that takes the persistent schedule). Exact data must match the oracle bit for bit, nothing may be
     stored past the end of C, and the reported plan is a tiled one."""
     assert rfk.select_config(m, n, k).variant >= 0
     data = exact_problem(m, n, k, seed=3 * m + 5 * n + k)
