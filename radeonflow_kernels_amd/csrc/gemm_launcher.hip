@@ -69,6 +69,7 @@ const Variant kVariants[] = {
     RF_VARIANT(128, 64, 2, 1),    // 4: 2 waves, wave tile 64 x 64, 48 KiB LDS (3 workgroups per CU)
     RF_VARIANT_TILE_ONLY(192, 192, 2, 4),   // 5: 8 waves, wave tile 96 x 48, 98 KiB LDS (6144 x 4608 = 768 tiles = 3 x 256)
     RF_VARIANT_TILE_ONLY(128, 192, 2, 4),   // 6: 8 waves, wave tile 64 x 48, 82 KiB LDS (N = 576, 1536: no padded columns)
+    RF_VARIANT_TILE_ONLY(64, 128, 2, 2),    // 7: 4 waves, wave tile 32 x 64, 49 KiB LDS (3 workgroups per CU; short M)
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
@@ -230,15 +231,16 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
         return;
     }
     // No measured entry: a cost model fitted to the tuner's measurements of the tabled shapes (on those its plan is
-    // 1.5 % slower than the best measured one on average, 14 % at worst). Time in microseconds of a plan =
+    // 2 % slower than the best measured one on average, 13 % at worst). Time in microseconds of a plan =
     //   rounds * (K blocks per workgroup * c + f)           one workgroup per tile and K split
     //   rounds * K blocks * c + f + (rounds - 1) * f_next   persistent: only the first tile starts cold
     //   + reduction cost when K is split
-    // with rounds = ceil(workgroups / CUs). Candidates: the 256x256, 128x256, 192x192 and 128x192 tiles (the last two
-    // win where they divide the shape into fuller rounds or leave no padded columns, e.g. N = 576, 1536 or 3072); the
-    // smaller ones never won by more than a few percent.
+    // with rounds = ceil(workgroups / CUs). Candidates: the 256x256, 128x256, 192x192, 128x192 and 64x128 tiles (192-wide
+    // tiles win where they divide the shape into fuller rounds or leave no padded columns, e.g. N = 576, 1536 or 3072;
+    // the 64x128 tile where M is short or the whole problem is a few microseconds); the others never won by more than
+    // a few percent.
     struct Candidate { int variant; double c, f; };
-    const Candidate cands[] = {{0, 1.355, 9.46}, {3, 0.769, 3.61}, {5, 0.95, 6.0}, {6, 0.65, 4.0}};
+    const Candidate cands[] = {{0, 1.355, 9.46}, {3, 0.769, 3.61}, {5, 0.95, 6.0}, {6, 0.65, 4.0}, {7, 0.55, 1.0}};
     const double f_next = 3.0, reduce_fixed = 6.83, reduce_per_elem = 8.7e-7;
     const int splits_tried[] = {1, 2, 3, 4, 6, 8, 12, 16};
     const int qk = k / rf::BK;
