@@ -16,7 +16,8 @@
  * pass over a; when N is ragged or c unaligned also one over b and a staged copy of c). Problems below 2^21 multiply-adds, and explicit plans with
  * variant = -1, take a bounds-checked kernel instead (the role of the reference's legacy kernel,
  * src/gemm/gemm_kernel_legacy.cpp:237-374).
- * Not thread-safe across host threads (one lazily grown workspace per process), like the reference.
+ * Workspace, staging buffer and counters exist once per device and belong to the device that is current at the call;
+ * calls are serialised by one lock, but launches that share a device's buffers must not overlap on different streams.
  */
 #ifndef RF_GEMM_H
 #define RF_GEMM_H
@@ -110,7 +111,7 @@ int rf_gemm_variant_has_persistent(int variant);
  * of ragged or unaligned operands are not part of it: that buffer grows on the first such call. */
 size_t rf_gemm_workspace_bytes(int m, int n, int k);
 
-/* Optional explicit set-up / tear-down of the process-wide workspace on the current device. run() and
+/* Optional explicit set-up / tear-down of the current device's workspace. run() and
  * rf_fp8_gemm() grow it lazily on first use (the reference's init_workspace, src/gemm/gemm_launcher.cpp:30-36,50-53,
  * allocates a fixed 1.5 GB instead). rf_gemm_init(bytes) pre-allocates so that later calls allocate nothing. */
 int rf_gemm_init(size_t workspace_bytes);

@@ -78,22 +78,33 @@ struct TunedPlan {
     int m, n, k, variant, split_k, group_m, stream_k;
 };
 
+// Buffers, counters and kernel attributes belong to a device: one State per device, chosen by the device that is
+// current at the call. Plans and the lock are shared by the process.
 struct State {
-    std::mutex mu;
     uint8_t *pad = nullptr;              // staging for shapes the tiled kernels do not take as they are (see launch_padded)
     size_t pad_bytes = 0;
-    std::vector<TunedPlan> user_plans;   // rf_gemm_load_plans / RF_GEMM_PLANS: looked up before the built-in table
-    bool env_plans_checked = false;
     float *ws = nullptr;
     size_t ws_bytes = 0;
     unsigned *tile_count = nullptr;      // stream-K arrival counters, zero between launches
-    bool attrs_set = false;
+    bool attrs_set = false, grouped_attrs_set = false;
     int num_cu = 0;
     std::vector<std::pair<hipEvent_t, hipEvent_t>> free_events;
 };
-State &state() {
-    static State s;
+struct Shared {
+    std::mutex mu;
+    std::vector<TunedPlan> user_plans;   // rf_gemm_load_plans / RF_GEMM_PLANS: looked up before the built-in table
+    bool env_plans_checked = false;
+};
+constexpr int kMaxDevices = 64;
+Shared &shared() {
+    static Shared s;
     return s;
+}
+State &state() {
+    static State states[kMaxDevices];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) dev = 0;
+    return states[dev];
 }
 
 // Plan file: one plan per line, "M N K variant split_k group_m stream_k"; braces and commas count as blanks (so a
@@ -131,13 +142,13 @@ int parse_plans(const char *path, std::vector<TunedPlan> &out) {
 
 int ensure_device_info(State &s) {
     if (s.attrs_set) return RF_OK;
-    if (!s.env_plans_checked) {
+    if (!shared().env_plans_checked) {
         // a file named by RF_GEMM_PLANS is loaded once, before the first plan is chosen; a bad file is an error
         if (const char *path = getenv("RF_GEMM_PLANS")) {
-            int rc = parse_plans(path, s.user_plans);
+            int rc = parse_plans(path, shared().user_plans);
             if (rc != RF_OK) return rc;
         }
-        s.env_plans_checked = true;
+        shared().env_plans_checked = true;
     }
     int dev = 0;
     RF_HIP(hipGetDevice(&dev));
@@ -295,7 +306,7 @@ int launch_locked(State &s, const void *a, const void *b, const float *as, const
             return fail(RF_ERR_BAD_CONFIG, "unknown schedule");
         }
     } else {
-        select_config(m, n, k, s.num_cu, tiled_ok, s.user_plans, &cfg);
+        select_config(m, n, k, s.num_cu, tiled_ok, shared().user_plans, &cfg);
     }
 
     if (m_store != m && (cfg.variant < 0 || cfg.stream_k != RF_SCHEDULE_TILES))
@@ -448,7 +459,7 @@ int launch_padded(State &s, const void *a, const void *b, const float *as, const
     // The plan of the padded shape. With whole columns and an aligned c, a plan of one workgroup per tile writes the m
     // true rows straight into c (its stores are masked by row); otherwise C is staged and copied back.
     rf_gemm_config cfg;
-    select_config(mp, np, k, s.num_cu, true, s.user_plans, &cfg);
+    select_config(mp, np, k, s.num_cu, true, shared().user_plans, &cfg);
     const bool copy_c = np != n || (uintptr_t)c % 16 != 0 || (mp != m && cfg.stream_k != RF_SCHEDULE_TILES);
     size_t off = 0;
     const size_t off_a = off;  off += copy_a ? align((size_t)k * mp) : 0;
@@ -492,7 +503,7 @@ int launch(const void *a, const void *b, const float *as, const float *bs, void 
                                           " K=" + std::to_string(k) + " (need M,N>=1, K a positive multiple of 128)");
     if (!a || !b || !as || !bs || !c) return fail(RF_ERR_NULL_POINTER, "null device pointer");
     State &s = state();
-    std::lock_guard<std::mutex> lock(s.mu);
+    std::lock_guard<std::mutex> lock(shared().mu);
     int rc = ensure_device_info(s);
     if (rc != RF_OK) return rc;
     if (!user_cfg && !tiled_path_ok(a, b, c, m, n) && (double)m * n * k >= kPadThresholdMacs)
@@ -505,6 +516,7 @@ struct TimerJob {
     hipEvent_t start, stop;
     double flop;
     float *time_ms, *gflops;
+    State *owner;                        // the device state whose event pool the pair came from
 };
 void timer_callback(hipStream_t, hipError_t status, void *user) {
     TimerJob *job = static_cast<TimerJob *>(user);
@@ -515,9 +527,9 @@ void timer_callback(hipStream_t, hipError_t status, void *user) {
             if (job->gflops) *job->gflops = (float)(job->flop / (ms * 1e-3) / 1e9);
         }
     }
-    State &s = state();
+    State &s = *job->owner;               // the callback thread has no current device of its own
     {
-        std::lock_guard<std::mutex> lock(s.mu);
+        std::lock_guard<std::mutex> lock(shared().mu);
         s.free_events.emplace_back(job->start, job->stop);   // recycled, unlike the reference's growing list
     }
     delete job;
@@ -570,7 +582,7 @@ int rf_gemm_select_config(int m, int n, int k, rf_gemm_config *out) {
     if (!out) return fail(RF_ERR_NULL_POINTER, "out is null");
     if (m < 1 || n < 1 || k < rf::BK || k % rf::BK != 0) return fail(RF_ERR_BAD_SHAPE, "unsupported shape");
     State &s = state();
-    std::lock_guard<std::mutex> lock(s.mu);
+    std::lock_guard<std::mutex> lock(shared().mu);
     int rc = ensure_device_info(s);
     if (rc != RF_OK) return rc;
     const bool tiled = m >= 16 && n >= 16 && m % 16 == 0 && n % 16 == 0;
@@ -578,29 +590,27 @@ int rf_gemm_select_config(int m, int n, int k, rf_gemm_config *out) {
         // the launch pads such a shape to multiples of 16 and plans for the padded shape (see launch_padded)
         m = m < 16 ? 16 : (m + 15) / 16 * 16;
         n = n < 16 ? 16 : (n + 15) / 16 * 16;
-        select_config(m, n, k, s.num_cu, true, s.user_plans, out);
+        select_config(m, n, k, s.num_cu, true, shared().user_plans, out);
         return RF_OK;
     }
-    select_config(m, n, k, s.num_cu, tiled, s.user_plans, out);
+    select_config(m, n, k, s.num_cu, tiled, shared().user_plans, out);
     return RF_OK;
 }
 
 int rf_gemm_load_plans(const char *path, int *count) {
     g_last_error.clear();
     if (!path) return fail(RF_ERR_NULL_POINTER, "path is null");
-    State &s = state();
-    std::lock_guard<std::mutex> lock(s.mu);
-    const size_t before = s.user_plans.size();
-    int rc = parse_plans(path, s.user_plans);
+    std::lock_guard<std::mutex> lock(shared().mu);
+    const size_t before = shared().user_plans.size();
+    int rc = parse_plans(path, shared().user_plans);
     if (rc != RF_OK) return rc;
-    if (count) *count = (int)(s.user_plans.size() - before);
+    if (count) *count = (int)(shared().user_plans.size() - before);
     return RF_OK;
 }
 
 void rf_gemm_clear_plans(void) {
-    State &s = state();
-    std::lock_guard<std::mutex> lock(s.mu);
-    s.user_plans.clear();
+    std::lock_guard<std::mutex> lock(shared().mu);
+    shared().user_plans.clear();
 }
 
 int rf_gemm_num_variants(void) { return kNumVariants; }
@@ -643,7 +653,7 @@ size_t rf_gemm_workspace_bytes(int m, int n, int k) {
 int rf_gemm_init(size_t workspace_bytes) {
     g_last_error.clear();
     State &s = state();
-    std::lock_guard<std::mutex> lock(s.mu);
+    std::lock_guard<std::mutex> lock(shared().mu);
     int rc = ensure_device_info(s);
     if (rc != RF_OK) return rc;
     return ensure_workspace(s, workspace_bytes);
@@ -651,7 +661,7 @@ int rf_gemm_init(size_t workspace_bytes) {
 
 void rf_gemm_destroy(void) {
     State &s = state();
-    std::lock_guard<std::mutex> lock(s.mu);
+    std::lock_guard<std::mutex> lock(shared().mu);
     if (s.ws) {
         (void)hipDeviceSynchronize();
         (void)hipFree(s.ws);
@@ -687,7 +697,7 @@ int launch_quantize(const void *x, int rows, int k, void *out, float *scales, hi
         return fail(RF_ERR_BAD_CONFIG, "source must be 16-byte aligned, scales 4-byte aligned");
     State &s = state();
     {
-        std::lock_guard<std::mutex> lock(s.mu);
+        std::lock_guard<std::mutex> lock(shared().mu);
         int rc = ensure_device_info(s);
         if (rc != RF_OK) return rc;
     }
@@ -721,7 +731,6 @@ const GroupedVariant kGroupedVariants[] = {
     GroupedVariant{256, 256, 512, rf::TileGeom<256, 256, 2, 4>::LDS_BYTES, rf::gemm_fp8_blockscale_grouped_mixed, true}};
 constexpr int kGroupedMixed = 4;
 constexpr int kNumGroupedVariants = sizeof(kGroupedVariants) / sizeof(kGroupedVariants[0]);
-bool g_grouped_attrs_set = false;
 
 long grouped_tiles(const GroupedVariant &v, const int *row_offsets, int groups, int n) {
     long t = 0;
@@ -747,13 +756,13 @@ int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const flo
     if (!a || !b || !as || !bs || !c) return fail(RF_ERR_NULL_POINTER, "null device pointer");
     if (variant >= kNumGroupedVariants || variant < -1) return fail(RF_ERR_BAD_CONFIG, "no such grouped variant");
     State &s = state();
-    std::lock_guard<std::mutex> lock(s.mu);
+    std::lock_guard<std::mutex> lock(shared().mu);
     int rc = ensure_device_info(s);
     if (rc != RF_OK) return rc;
-    if (!g_grouped_attrs_set) {
+    if (!s.grouped_attrs_set) {
         for (const GroupedVariant &v : kGroupedVariants)
             RF_HIP(hipFuncSetAttribute((const void *)v.kernel, hipFuncAttributeMaxDynamicSharedMemorySize, v.lds));
-        g_grouped_attrs_set = true;
+        s.grouped_attrs_set = true;
     }
     const int qk = k / rf::BK, qn = ceil_div(n, 128);
     const bool direct = n % 16 == 0 && ((uintptr_t)b % 16) == 0 && ((uintptr_t)c % 16) == 0;
@@ -873,8 +882,9 @@ void run(void *a, void *b, void *as, void *bs, void *c, int m, int n, int k, Per
     if (metrics) {
         job = new TimerJob();
         State &s = state();
+        job->owner = &s;
         {
-            std::lock_guard<std::mutex> lock(s.mu);
+            std::lock_guard<std::mutex> lock(shared().mu);
             if (!s.free_events.empty()) {
                 job->start = s.free_events.back().first;
                 job->stop = s.free_events.back().second;
