@@ -408,3 +408,29 @@ def test_hip_graph_replays_match_eager(rfk):
         step(xs[(i + 1) % 4], again)
         torch.cuda.synchronize()
         assert torch.equal(again[1].view(torch.uint16), eager[(i + 1) % 4][1].view(torch.uint16))
+
+
+def test_operand_beyond_2_gib_is_addressed_with_64_bits(rfk):
+    """A of more than 2^31 bytes: rows near the end are reached only if every index is computed in 64 bits. Values in
+    {0, +-1} and scales in {0.5, 1, 2} keep every sum exact in fp32, so sampled rows must match the oracle bit for bit."""
+    m, n, k = 163840, 256, 13312
+    assert m * k > 2 ** 31
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev).manual_seed(11)
+    codes = torch.tensor([0x00, 0x38, 0xB8, 0x38], dtype=torch.uint8, device=dev)
+    a8 = codes[torch.randint(0, 4, (k, m), device=dev, generator=gen)]
+    b8 = codes[torch.randint(0, 4, (k, n), device=dev, generator=gen)]
+    pow2 = torch.tensor([0.5, 1.0, 2.0], device=dev)
+    sa = pow2[torch.randint(0, 3, (k // 128, m), device=dev, generator=gen)]
+    sb = pow2[torch.randint(0, 3, (k // 128, n // 128), device=dev, generator=gen)]
+    c = torch.zeros((m, n), dtype=torch.bfloat16, device=dev)
+    fp8 = torch.float8_e4m3fn
+    rows = np.unique(np.concatenate([[0, 1, 77, m // 2, m - 17, m - 1],
+                                     np.random.default_rng(5).integers(0, m, 26)])).astype(np.int32)
+    exp = cref.ref_gemm_blockfold(a8.cpu().numpy(), b8.cpu().numpy(), sa.cpu().numpy(), sb.cpu().numpy(), rows=rows)[1]
+    for cfg in (None, rfk.GemmConfig(3, 1, 8, 0), rfk.GemmConfig(0, 2, 4, 0)):
+        c.zero_()
+        rfk.fp8_mm(a8.view(fp8).T, b8.view(fp8).T, sa.T, sb.T, c, config=cfg)
+        torch.cuda.synchronize()
+        got = bf16_bits(c[torch.from_numpy(rows.astype(np.int64)).to(dev)])
+        assert np.array_equal(got, exp), "plan %r" % (cfg,)

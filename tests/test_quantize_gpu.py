@@ -177,3 +177,24 @@ def test_status_codes(rfk):
     assert L.rf_quantize_a_f32(x.data_ptr(), 128, 100, q.data_ptr(), s.data_ptr(), None) == 1     # RF_ERR_BAD_SHAPE
     assert L.rf_quantize_a_f32(None, 128, 128, q.data_ptr(), s.data_ptr(), None) == 2            # RF_ERR_NULL_POINTER
     assert L.rf_quantize_a_f32(x.data_ptr() + 4, 127, 128, q.data_ptr(), s.data_ptr(), None) == 4  # misaligned source
+
+
+def test_quantize_a_source_beyond_4_gib(rfk):
+    """A source of more than 2^32 bytes (and more than 2^31 elements of output index range per K row times rows):
+    sampled rows, the last ones included, against the oracle's quantiser run on those rows alone (a row's scales and
+    codes depend on nothing but the row)."""
+    rows, k = 163840, 7168
+    assert rows * k * 4 > 2 ** 32
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev).manual_seed(3)
+    x = torch.randn((rows, k), device=dev, generator=gen)
+    q, s = rfk.quantize_a(x)
+    torch.cuda.synchronize()
+    pick = np.unique(np.concatenate([[0, 1, 127, 128, rows // 2, rows - 129, rows - 2, rows - 1],
+                                     np.random.default_rng(9).integers(0, rows, 24)]))
+    idx = torch.from_numpy(pick).to(dev)
+    a_ref, as_ref = cref.quantize_a(np.ascontiguousarray(x[idx].cpu().numpy()))        # [K][len(pick)], [K/128][len(pick)]
+    got_codes = q[idx].contiguous().view(torch.uint8).cpu().numpy().T                   # q is [rows, K] stride (1, rows)
+    got_scales = s[idx].contiguous().cpu().numpy().T
+    assert np.array_equal(got_scales.view(np.uint32), np.asarray(as_ref).view(np.uint32))
+    assert np.array_equal(got_codes, np.asarray(a_ref))
