@@ -735,10 +735,31 @@ __global__ __launch_bounds__(256) void reduce_splitk_bf16(const float *__restric
                                                           size_t mn, int splits, size_t split_stride) {
     size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= mn) return;
-    f32x4 s = *(const f32x4 *)(ws + i);
-    for (int p = 1; p < splits; p++) {
-        f32x4 v = *(const f32x4 *)(ws + (size_t)p * split_stride + i);
-        s[0] += v[0]; s[1] += v[1]; s[2] += v[2]; s[3] += v[3];
+    const float *p = ws + i;
+    f32x4 s = *(const f32x4 *)p;
+    // The partials of up to 8 splits are fetched together and then added in split order: with one load per loop
+    // iteration a small output (few threads, nothing else to run) pays the memory latency once per split.
+    constexpr int BATCH = 8;
+    int q0 = 1;
+    for (; q0 + BATCH <= splits; q0 += BATCH) {
+        f32x4 v[BATCH];
+#pragma unroll
+        for (int q = 0; q < BATCH; q++) v[q] = *(const f32x4 *)(p + (size_t)(q0 + q) * split_stride);
+#pragma unroll
+        for (int q = 0; q < BATCH; q++) {
+            s[0] += v[q][0]; s[1] += v[q][1]; s[2] += v[q][2]; s[3] += v[q][3];
+        }
+    }
+    if (q0 < splits) {
+        f32x4 v[BATCH - 1];
+#pragma unroll
+        for (int q = 0; q < BATCH - 1; q++)
+            if (q0 + q < splits) v[q] = *(const f32x4 *)(p + (size_t)(q0 + q) * split_stride);
+#pragma unroll
+        for (int q = 0; q < BATCH - 1; q++)
+            if (q0 + q < splits) {
+                s[0] += v[q][0]; s[1] += v[q][1]; s[2] += v[q][2]; s[3] += v[q][3];
+            }
     }
     uint2 o;
     o.x = pack_bf16x2(s[0], s[1]);
