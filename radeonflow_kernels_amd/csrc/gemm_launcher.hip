@@ -394,47 +394,79 @@ int ensure_pad(State &s, size_t bytes) {
 // The grouped GEMM's staging copy: the caller's [rows][m_total] matrix (A with T = bytes, a_scale with T = float), in
 // which group g owns columns out_row_start[g] .. out_row_start[g+1]-1, is copied to [rows][m_pad] with group g starting
 // at column row_start[g], a multiple of 16; the columns between a group's end and the next start become zero.
-// blockIdx.y is the group, so the table is read with uniform indices; every thread writes aligned 16-byte pieces.
-// Bytes are fetched as the aligned words that hold them and shifted into place: a source piece starts at any byte.
+// A workgroup writes 256 consecutive 16-byte pieces of kPadRows consecutive rows, whatever groups they belong to, so
+// both sides of the copy move whole cache lines even when the groups are a few rows each. The groups that overlap the
+// workgroup's columns are found with uniform (scalar) reads of the table; each thread then keeps the last one that
+// starts at or before its column. Bytes are fetched as the aligned words that hold them and shifted into place: a
+// source piece starts at any byte.
+constexpr int kPadRows = 4;
 template <typename T>
 __global__ __launch_bounds__(256) void pad_group_rows(const T *__restrict__ src, int m_total, int m_pad, int rows,
-                                                      T *__restrict__ dst, const rf::GroupTable table) {
+                                                      int groups, T *__restrict__ dst, const rf::GroupTable table) {
     constexpr int PER = 16 / sizeof(T);
-    const int g = blockIdx.y, start = table.row_start[g], pieces = (table.row_start[g + 1] - start) / PER;
-    const int from = table.out_row_start[g], count = table.out_row_start[g + 1] - from;
-    const long work = (long)pieces * rows;
-    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < work; i += (long)gridDim.x * 256) {
-        const int r = (int)(i / pieces), col = (int)(i % pieces) * PER;
-        int valid = count - col;                                       // columns of this piece that exist in the source
-        valid = valid < 0 ? 0 : valid > PER ? PER : valid;
-        const T *p = src + (size_t)r * m_total + from + col;
+    const int c_lo = blockIdx.y * 256 * PER, c_hi = (c_lo + 256 * PER < m_pad ? c_lo + 256 * PER : m_pad) - 1;
+    auto last_group_starting_by = [&](int c) {                       // uniform binary search
+        int lo = 0, hi = groups;
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (table.row_start[mid] <= c) lo = mid; else hi = mid;
+        }
+        return lo;
+    };
+    const int g_lo = last_group_starting_by(c_lo), g_hi = last_group_starting_by(c_hi);
+    const int col = c_lo + (int)threadIdx.x * PER;
+    int start = table.row_start[g_lo], from = table.out_row_start[g_lo], count = table.out_row_start[g_lo + 1] - from;
+    for (int g = g_lo + 1; g <= g_hi; g++) {
+        const int s2 = table.row_start[g], f2 = table.out_row_start[g], n2 = table.out_row_start[g + 1] - f2;
+        if (col >= s2) { start = s2; from = f2; count = n2; }
+    }
+    if (col >= m_pad) return;
+    int valid = count - (col - start);                                 // columns of this piece that exist in the source
+    valid = valid < 0 ? 0 : valid > PER ? PER : valid;
+    const int r_first = blockIdx.x * kPadRows;
+    const T *p0 = src + (size_t)r_first * m_total + from + (col - start);
+    uint32_t w[kPadRows][5];
+    int shift[kPadRows];
+#pragma unroll
+    for (int u = 0; u < kPadRows; u++) {
+        const T *p = p0 + (size_t)u * m_total;
+        shift[u] = 0;
+        if (r_first + u < rows) {
+            if constexpr (sizeof(T) == 4) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) w[u][e] = e < valid ? ((const uint32_t *)p)[e] : 0u;
+            } else {
+                shift[u] = (int)((uintptr_t)p & 3);
+                const int need = valid ? shift[u] + valid : 0;
+                const uint32_t *q = (const uint32_t *)((const uint8_t *)p - shift[u]);
+#pragma unroll
+                for (int e = 0; e < 5; e++) w[u][e] = 4 * e < need ? q[e] : 0u;   // only words that hold a wanted byte
+            }
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kPadRows; u++) {
+        if (r_first + u >= rows) continue;
         uint32_t out[4];
         if constexpr (sizeof(T) == 4) {
 #pragma unroll
-            for (int e = 0; e < 4; e++) out[e] = e < valid ? ((const uint32_t *)p)[e] : 0u;
+            for (int e = 0; e < 4; e++) out[e] = w[u][e];
         } else {
-            const int shift = (int)((uintptr_t)p & 3), need = valid ? shift + valid : 0;
-            const uint32_t *q = (const uint32_t *)((const uint8_t *)p - shift);
-            uint32_t w[5];
-#pragma unroll
-            for (int e = 0; e < 5; e++) w[e] = 4 * e < need ? q[e] : 0u;   // only words that hold a wanted byte
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                out[e] = __builtin_amdgcn_alignbyte(w[e + 1], w[e], shift);
+                out[e] = __builtin_amdgcn_alignbyte(w[u][e + 1], w[u][e], shift[u]);
                 const int nv = valid - 4 * e;
                 if (nv < 4) out[e] = nv <= 0 ? 0u : out[e] & ((1u << (8 * nv)) - 1u);
             }
         }
-        *(uint4 *)(dst + (size_t)r * m_pad + start + col) = make_uint4(out[0], out[1], out[2], out[3]);
+        *(uint4 *)(dst + (size_t)(r_first + u) * m_pad + col) = make_uint4(out[0], out[1], out[2], out[3]);
     }
 }
 
-// grid of pad_group_rows: enough workgroups for one piece per thread, capped (threads loop over the rest)
-dim3 pad_grid(long pieces_of_largest_group, int groups) {
-    long x = (pieces_of_largest_group + 255) / 256;
-    const long cap = 4096 / groups > 0 ? 4096 / groups : 1;
-    x = x < 1 ? 1 : x > cap ? cap : x;
-    return dim3((unsigned)x, (unsigned)groups);
+// grid of pad_group_rows for `rows` rows of m_pad elements of `size` bytes
+dim3 pad_grid(int m_pad, int size, int rows) {
+    const int pieces = m_pad / (16 / size);
+    return dim3((unsigned)((rows + kPadRows - 1) / kPadRows), (unsigned)((pieces + 255) / 256));     // rows on x: no 65535 limit
 }
 
 // table of one group of `cols` columns padded to `cols_pad`
@@ -472,17 +504,17 @@ int launch_padded(State &s, const void *a, const void *b, const float *as, const
     const float *as2 = as;
     void *c2 = c;
     if (copy_a) {
-        hipLaunchKernelGGL(pad_group_rows<uint8_t>, pad_grid((long)k * (mp / 16), 1), dim3(256), 0, stream,
-                           (const uint8_t *)a, m, mp, k, s.pad + off_a, one_group(m, mp));
+        hipLaunchKernelGGL(pad_group_rows<uint8_t>, pad_grid(mp, 1, k), dim3(256), 0, stream, (const uint8_t *)a, m, mp, k, 1,
+                           s.pad + off_a, one_group(m, mp));
         a2 = s.pad + off_a;
     }
     if (copy_b) {
-        hipLaunchKernelGGL(pad_group_rows<uint8_t>, pad_grid((long)k * (np / 16), 1), dim3(256), 0, stream,
-                           (const uint8_t *)b, n, np, k, s.pad + off_b, one_group(n, np));
+        hipLaunchKernelGGL(pad_group_rows<uint8_t>, pad_grid(np, 1, k), dim3(256), 0, stream, (const uint8_t *)b, n, np, k, 1,
+                           s.pad + off_b, one_group(n, np));
         b2 = s.pad + off_b;
     }
     if (copy_sa) {
-        hipLaunchKernelGGL(pad_group_rows<float>, pad_grid((long)qk * (mp / 4), 1), dim3(256), 0, stream, as, m, mp, qk,
+        hipLaunchKernelGGL(pad_group_rows<float>, pad_grid(mp, 4, qk), dim3(256), 0, stream, as, m, mp, qk, 1,
                            (float *)(s.pad + off_sa), one_group(m, mp));
         as2 = (const float *)(s.pad + off_sa);
     }
@@ -790,12 +822,10 @@ int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const flo
         // each group's true rows straight into the caller's C. Costs one pass over A; the bounds-checked kernel
         // per group would be 10 to 30 times slower than the tiled one.
         int at = 0;
-        long most = 0;
         for (int g = 0; g < groups; g++) {
             table.row_start[g] = at;
             const int pr = (row_offsets[g + 1] - row_offsets[g] + 15) / 16 * 16;
             at += pr;
-            most = pr > most ? pr : most;
         }
         for (int g = groups; g <= rf::kMaxGroups; g++) table.row_start[g] = at;
         for (int g = 0; g <= rf::kMaxGroups; g++) table.out_row_start[g] = row_offsets[g < groups ? g : groups];
@@ -803,10 +833,10 @@ int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const flo
         const size_t a_bytes = ((size_t)k * m_rows + 255) / 256 * 256;
         rc = ensure_pad(s, a_bytes + (size_t)qk * m_rows * sizeof(float));
         if (rc != RF_OK) return rc;
-        hipLaunchKernelGGL(pad_group_rows<uint8_t>, pad_grid(most / 16 * k, groups), dim3(256), 0, stream,
-                           (const uint8_t *)a, m_total, m_rows, k, s.pad, table);
-        hipLaunchKernelGGL(pad_group_rows<float>, pad_grid(most / 4 * qk, groups), dim3(256), 0, stream, as, m_total,
-                           m_rows, qk, (float *)(s.pad + a_bytes), table);
+        hipLaunchKernelGGL(pad_group_rows<uint8_t>, pad_grid(m_rows, 1, k), dim3(256), 0, stream, (const uint8_t *)a,
+                           m_total, m_rows, k, groups, s.pad, table);
+        hipLaunchKernelGGL(pad_group_rows<float>, pad_grid(m_rows, 4, qk), dim3(256), 0, stream, as, m_total, m_rows, qk,
+                           groups, (float *)(s.pad + a_bytes), table);
         RF_HIP(hipGetLastError());
         a = s.pad;
         as = (const float *)(s.pad + a_bytes);
