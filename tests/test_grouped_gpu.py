@@ -90,7 +90,8 @@ def test_grouped_ragged_n_or_tiny_problems_take_the_checked_kernel(rfk, rows, n,
 
 
 RAGGED = [([5, 17, 0, 100, 333, 1], 512, 256), ([1, 1, 1, 1, 300], 256, 384), ([255, 257, 129, 0, 143, 15], 768, 256),
-          ([1000], 256, 128), ([int(x) for x in np.random.default_rng(3).integers(0, 300, 40)], 576, 256)]
+          ([1000], 256, 128), ([int(x) for x in np.random.default_rng(3).integers(0, 300, 40)], 576, 256),
+          ([int(x) for x in np.random.default_rng(4).integers(0, 21, 256)], 256, 128)]      # 256 groups of 0..20 rows
 
 
 @pytest.mark.parametrize("rows,n,k", RAGGED)
