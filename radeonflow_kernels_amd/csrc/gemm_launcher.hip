@@ -401,10 +401,12 @@ int ensure_pad(State &s, size_t bytes) {
 // source piece starts at any byte.
 constexpr int kPadRows = 4;
 template <typename T>
-__global__ __launch_bounds__(256) void pad_group_rows(const T *__restrict__ src, int m_total, int m_pad, int rows,
-                                                      int groups, T *__restrict__ dst, const rf::GroupTable table) {
+__device__ __forceinline__ void pad_group_rows_body(const T *__restrict__ src, int m_total, int m_pad, int rows, int groups,
+                                                    T *__restrict__ dst, const rf::GroupTable &table, int block_row,
+                                                    int block_chunk) {
     constexpr int PER = 16 / sizeof(T);
-    const int c_lo = blockIdx.y * 256 * PER, c_hi = (c_lo + 256 * PER < m_pad ? c_lo + 256 * PER : m_pad) - 1;
+    if (block_chunk * 256 * PER >= m_pad) return;
+    const int c_lo = block_chunk * 256 * PER, c_hi = (c_lo + 256 * PER < m_pad ? c_lo + 256 * PER : m_pad) - 1;
     auto last_group_starting_by = [&](int c) {                       // uniform binary search
         int lo = 0, hi = groups;
         while (hi - lo > 1) {
@@ -423,7 +425,7 @@ __global__ __launch_bounds__(256) void pad_group_rows(const T *__restrict__ src,
     if (col >= m_pad) return;
     int valid = count - (col - start);                                 // columns of this piece that exist in the source
     valid = valid < 0 ? 0 : valid > PER ? PER : valid;
-    const int r_first = blockIdx.x * kPadRows;
+    const int r_first = block_row * kPadRows;
     const T *p0 = src + (size_t)r_first * m_total + from + (col - start);
     uint32_t w[kPadRows][5];
     int shift[kPadRows];
@@ -463,10 +465,36 @@ __global__ __launch_bounds__(256) void pad_group_rows(const T *__restrict__ src,
     }
 }
 
+template <typename T>
+__global__ __launch_bounds__(256) void pad_group_rows(const T *__restrict__ src, int m_total, int m_pad, int rows,
+                                                      int groups, T *__restrict__ dst, const rf::GroupTable table) {
+    pad_group_rows_body<T>(src, m_total, m_pad, rows, groups, dst, table, blockIdx.x, blockIdx.y);
+}
+
+// A and a_scale in one launch (they are staged together whenever M or the group sizes are ragged): the first
+// blocks_a workgroups along x copy the bytes of A, the others the floats of a_scale.
+__global__ __launch_bounds__(256) void pad_group_rows_a_and_scales(const uint8_t *__restrict__ a, const float *__restrict__ as,
+                                                                   int m_total, int m_pad, int k, int groups,
+                                                                   uint8_t *__restrict__ a_dst, float *__restrict__ as_dst,
+                                                                   int blocks_a, const rf::GroupTable table) {
+    if ((int)blockIdx.x < blocks_a)
+        pad_group_rows_body<uint8_t>(a, m_total, m_pad, k, groups, a_dst, table, blockIdx.x, blockIdx.y);
+    else
+        pad_group_rows_body<float>(as, m_total, m_pad, k / rf::BK, groups, as_dst, table, blockIdx.x - blocks_a, blockIdx.y);
+}
+
 // grid of pad_group_rows for `rows` rows of m_pad elements of `size` bytes
 dim3 pad_grid(int m_pad, int size, int rows) {
     const int pieces = m_pad / (16 / size);
     return dim3((unsigned)((rows + kPadRows - 1) / kPadRows), (unsigned)((pieces + 255) / 256));     // rows on x: no 65535 limit
+}
+
+// Stages A and a_scale with one launch.
+void launch_pad_a_and_scales(const void *a, const float *as, int m_total, int m_pad, int k, int groups, uint8_t *a_dst,
+                             float *as_dst, const rf::GroupTable &table, hipStream_t stream) {
+    const dim3 ga = pad_grid(m_pad, 1, k), gs = pad_grid(m_pad, 4, k / rf::BK);
+    hipLaunchKernelGGL(pad_group_rows_a_and_scales, dim3(ga.x + gs.x, ga.y > gs.y ? ga.y : gs.y), dim3(256), 0, stream,
+                       (const uint8_t *)a, as, m_total, m_pad, k, groups, a_dst, as_dst, (int)ga.x, table);
 }
 
 // table of one group of `cols` columns padded to `cols_pad`
@@ -503,7 +531,11 @@ int launch_padded(State &s, const void *a, const void *b, const float *as, const
     const void *a2 = a, *b2 = b;
     const float *as2 = as;
     void *c2 = c;
-    if (copy_a) {
+    if (copy_a && copy_sa) {
+        launch_pad_a_and_scales(a, as, m, mp, k, 1, s.pad + off_a, (float *)(s.pad + off_sa), one_group(m, mp), stream);
+        a2 = s.pad + off_a;
+        as2 = (const float *)(s.pad + off_sa);
+    } else if (copy_a) {                                   // M is fine, only the pointer is not aligned
         hipLaunchKernelGGL(pad_group_rows<uint8_t>, pad_grid(mp, 1, k), dim3(256), 0, stream, (const uint8_t *)a, m, mp, k, 1,
                            s.pad + off_a, one_group(m, mp));
         a2 = s.pad + off_a;
@@ -512,11 +544,6 @@ int launch_padded(State &s, const void *a, const void *b, const float *as, const
         hipLaunchKernelGGL(pad_group_rows<uint8_t>, pad_grid(np, 1, k), dim3(256), 0, stream, (const uint8_t *)b, n, np, k, 1,
                            s.pad + off_b, one_group(n, np));
         b2 = s.pad + off_b;
-    }
-    if (copy_sa) {
-        hipLaunchKernelGGL(pad_group_rows<float>, pad_grid(mp, 4, qk), dim3(256), 0, stream, as, m, mp, qk, 1,
-                           (float *)(s.pad + off_sa), one_group(m, mp));
-        as2 = (const float *)(s.pad + off_sa);
     }
     if (copy_c) c2 = s.pad + off_c;
     RF_HIP(hipGetLastError());
@@ -833,10 +860,7 @@ int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const flo
         const size_t a_bytes = ((size_t)k * m_rows + 255) / 256 * 256;
         rc = ensure_pad(s, a_bytes + (size_t)qk * m_rows * sizeof(float));
         if (rc != RF_OK) return rc;
-        hipLaunchKernelGGL(pad_group_rows<uint8_t>, pad_grid(m_rows, 1, k), dim3(256), 0, stream, (const uint8_t *)a,
-                           m_total, m_rows, k, groups, s.pad, table);
-        hipLaunchKernelGGL(pad_group_rows<float>, pad_grid(m_rows, 4, qk), dim3(256), 0, stream, as, m_total, m_rows, qk,
-                           groups, (float *)(s.pad + a_bytes), table);
+        launch_pad_a_and_scales(a, as, m_total, m_rows, k, groups, s.pad, (float *)(s.pad + a_bytes), table, stream);
         RF_HIP(hipGetLastError());
         a = s.pad;
         as = (const float *)(s.pad + a_bytes);
