@@ -434,3 +434,26 @@ def test_operand_beyond_2_gib_is_addressed_with_64_bits(rfk):
         torch.cuda.synchronize()
         got = bf16_bits(c[torch.from_numpy(rows.astype(np.int64)).to(dev)])
         assert np.array_equal(got, exp), "plan %r" % (cfg,)
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 384, 512), (1024, 576, 1024), (100, 130, 256)])
+def test_signed_zeros_and_negative_scales(rfk, m, n, k):
+    """Rows of -0 and +0 codes and rows with negative scales (the reference draws signed scales,
+    tests/gemm/gemm_test.cpp:90-92): sums of signed zeros must come out as the oracle's +0, bit for bit, under every plan."""
+    a, b, sa, sb, c = exact_problem(m, n, k, seed=5)
+    a8, b8 = a.view(torch.uint8).clone(), b.view(torch.uint8).clone()
+    a8[0:m:3, :] = 0x80
+    a8[1:m:7, :] = 0x00
+    b8[0:n:5, :] = 0x80
+    sa = sa.clone()
+    sa[2:m:4, :] *= -1.0
+    data = (a8.view(torch.float8_e4m3fn), b8.view(torch.float8_e4m3fn), sa, sb, c)
+    exp = oracle_bf16(data)
+    plans = [None]
+    if m % 16 == 0 and n % 16 == 0:
+        plans += [rfk.GemmConfig(v["variant"], s, 4, 0) for v in rfk.variants() for s in (1, 2, 4) if s <= k // 128]
+        plans += [rfk.GemmConfig(v["variant"], 1, 4, 2) for v in rfk.variants()
+                  if v["persistent"] and m % v["block_m"] == 0 and n % v["block_n"] == 0 and (k // 128) % 2 == 0]
+    for cfg in plans:
+        out = _run(rfk, data, config=cfg)
+        assert np.array_equal(bf16_bits(out), exp), "plan %r" % (cfg,)
