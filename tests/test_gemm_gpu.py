@@ -457,3 +457,29 @@ def test_signed_zeros_and_negative_scales(rfk, m, n, k):
     for cfg in plans:
         out = _run(rfk, data, config=cfg)
         assert np.array_equal(bf16_bits(out), exp), "plan %r" % (cfg,)
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 384, 512), (1024, 576, 1024), (100, 130, 256)])
+def test_nan_codes_poison_their_row_or_column_only(rfk, m, n, k):
+    """e4m3fn NaN codes (0x7f, 0xff) in A make the whole output row NaN, in B the whole column, exactly where the oracle
+    has NaN (the reference's checker requires NaN positions to match, tests/checker/checker.cpp:10-105); everything else
+    stays bit-exact."""
+    a, b, sa, sb, c = exact_problem(m, n, k, seed=6)
+    a8, b8 = a.view(torch.uint8).clone(), b.view(torch.uint8).clone()
+    a8[5, 17] = 0x7F
+    a8[m - 1, k - 1] = 0xFF
+    b8[3, k // 2] = 0x7F
+    data = (a8.view(torch.float8_e4m3fn), b8.view(torch.float8_e4m3fn), sa, sb, c)
+    exp = oracle_bf16(data)
+    exp_nan = (exp & 0x7FFF) > 0x7F80
+    assert exp_nan[5].all() and exp_nan[m - 1].all() and exp_nan[:, 3].all() and exp_nan.sum() == 2 * n + m - 2
+    plans = [None]
+    if m % 16 == 0 and n % 16 == 0:
+        plans += [rfk.GemmConfig(v["variant"], s, 4, 0) for v in rfk.variants() for s in (1, 3) if s <= k // 128]
+        plans += [rfk.GemmConfig(v["variant"], 1, 4, 2) for v in rfk.variants()
+                  if v["persistent"] and m % v["block_m"] == 0 and n % v["block_n"] == 0 and (k // 128) % 2 == 0]
+    for cfg in plans:
+        got = bf16_bits(_run(rfk, data, config=cfg))
+        got_nan = (got & 0x7FFF) > 0x7F80
+        assert np.array_equal(got_nan, exp_nan), "NaN positions, plan %r" % (cfg,)
+        assert np.array_equal(got[~exp_nan], exp[~exp_nan]), "plan %r" % (cfg,)
