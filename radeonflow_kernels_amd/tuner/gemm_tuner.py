@@ -6,8 +6,9 @@ DISPATCH_GEMM(...) line. Here nothing is recompiled: every kernel variant is alr
 (variant, split_k, group_m) is passed to rf_fp8_gemm_ex at run time, so a sweep is a loop of timed launches.
 
   python -m radeonflow_kernels_amd.tuner.gemm_tuner --M 6144 --N 4608 --K 7168        one shape
-  python -m radeonflow_kernels_amd.tuner.gemm_tuner --all --emit                       every known shape, then
-                                                                                       rewrite csrc/tuned_plans.inc
+  python -m radeonflow_kernels_amd.tuner.gemm_tuner --all [--extended] --emit          every known shape (and M = 16 ...
+                                                                                       8192 for each of their (N, K)),
+                                                                                       then rewrite csrc/tuned_plans.inc
   python -m radeonflow_kernels_amd.tuner.gemm_tuner --M .. --N .. --K .. --emit-file my.plans
                                                   append the winner to a plan file: rf_gemm_load_plans(path) or the
                                                   environment variable RF_GEMM_PLANS uses it without a rebuild
@@ -33,6 +34,10 @@ SHAPES = [
     (64, 64, 128), (64, 1536, 7168), (64, 3072, 1536), (64, 576, 7168), (96, 7168, 256), (96, 7168, 2048),
     (96, 4608, 7168), (128, 7168, 2304), (128, 512, 7168), (512, 4096, 512), (512, 1536, 7168),
 ]
+# token counts a server sees, over the (N, K) pairs of the shapes above (--extended)
+EXTENDED_M = (16, 32, 64, 128, 256, 512, 1024, 2048, 4096, 8192)
+EXTENDED = [(m, n, k) for (n, k) in sorted({(n, k) for _, n, k in SHAPES if (n, k) != (64, 128)}) for m in EXTENDED_M
+            if (m, n, k) not in SHAPES]
 SPLITS = (1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 16)
 GROUPS = (4, 8, 16)
 
@@ -94,7 +99,7 @@ def tune_shape(rfk, m, n, k, log=print):
 
 
 def emit_plans(results, path=PLANS_INC):
-    lines = ["// Generated by radeonflow_kernels_amd/tuner/gemm_tuner.py --all --emit on one MI355X; do not edit by hand.",
+    lines = ["// Generated by radeonflow_kernels_amd/tuner/gemm_tuner.py --all [--extended] --emit on one MI355X; do not edit by hand.",
              "// {M, N, K, variant, split_k, group_m, stream_k},   best time, TFLOP/s"]
     for (m, n, k), cands in results.items():
         if not cands:
@@ -112,14 +117,16 @@ def main():
     ap.add_argument("--N", type=int)
     ap.add_argument("--K", type=int)
     ap.add_argument("--all", action="store_true")
-    ap.add_argument("--emit", action="store_true", help="rewrite csrc/tuned_plans.inc (rebuild libgemm.so afterwards)")
+    ap.add_argument("--extended", action="store_true", help="with --all: also M = 16 ... 8192 for every (N, K) of the list")
+    ap.add_argument("--emit", nargs="?", const=PLANS_INC, default=None, metavar="PATH",
+                    help="rewrite csrc/tuned_plans.inc, or PATH if given (rebuild libgemm.so afterwards)")
     ap.add_argument("--emit-file", default=None, help="append the best plan of every tuned shape to this plan file")
     ap.add_argument("--out", default=None)
     a = ap.parse_args()
     sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
     import radeonflow_kernels_amd as rfk
     rfk.lib()
-    shapes = SHAPES if a.all else [(a.M, a.N, a.K)]
+    shapes = (SHAPES + (EXTENDED if a.extended else [])) if a.all else [(a.M, a.N, a.K)]
     results = {}
     for (m, n, k) in shapes:
         cands = tune_shape(rfk, m, n, k)
@@ -136,8 +143,8 @@ def main():
             with open(os.path.join(a.out, "gemm_%dx%dx%d.json" % (m, n, k)), "w") as f:
                 json.dump(cands, f, indent=1)
     if a.emit:
-        emit_plans(results)
-        print("wrote", PLANS_INC)
+        emit_plans(results, a.emit)
+        print("wrote", a.emit)
     if a.emit_file:
         with open(a.emit_file, "a") as f:
             for (m, n, k), cands in results.items():
