@@ -131,3 +131,22 @@ def test_plan_files_parse_without_a_device(tmp_path):
         assert L.rf_gemm_load_plans(None, None) == 2
     finally:
         gemm.clear_plans()
+
+
+def test_compiled_in_plan_table_only_holds_plans_its_shapes_can_run():
+    """Every line of csrc/tuned_plans.inc names an existing variant, a split that leaves every part at least one K
+    block, and the persistent schedule only where the tile divides the shape and K/128 is even (a plan that cannot
+    run is skipped at lookup, so a bad line would silently fall back to the cost model)."""
+    from radeonflow_kernels_amd import gemm
+    L = gemm.lib()
+    inc = os.path.join(ROOT, "radeonflow_kernels_amd", "csrc", "tuned_plans.inc")
+    plans = [tuple(int(x) for x in re.findall(r"-?\d+", l.split("}")[0])) for l in open(inc) if l.startswith("{")]
+    assert len(plans) >= 29 and len(set(p[:3] for p in plans)) == len(plans)        # one plan per shape
+    for m, n, k, variant, split, group, schedule in plans:
+        bm, bn = ctypes.c_int(), ctypes.c_int()
+        assert L.rf_gemm_variant_info(variant, ctypes.byref(bm), ctypes.byref(bn), None, None, None) == 0
+        assert m % 16 == 0 and n % 16 == 0 and k % 128 == 0 and 1 <= split <= k // 128 and group >= 1
+        assert schedule in (0, 2), "the stream-K schedule is never tabled"
+        if schedule == 2:
+            assert L.rf_gemm_variant_has_persistent(variant) == 1 and split == 1
+            assert m % bm.value == 0 and n % bn.value == 0 and (k // 128) % 2 == 0
