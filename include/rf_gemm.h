@@ -16,8 +16,11 @@
  * pass over a; when N is ragged or c unaligned also one over b and a staged copy of c). Problems below 2^21 multiply-adds, and explicit plans with
  * variant = -1, take a bounds-checked kernel instead (the role of the reference's legacy kernel,
  * src/gemm/gemm_kernel_legacy.cpp:237-374).
- * Workspace, staging buffer and counters exist once per device and belong to the device that is current at the call;
- * calls are serialised by one lock, but launches that share a device's buffers must not overlap on different streams.
+ * Temporary device memory (split-K partial sums, staging copies, stream-K counters) is kept per (device, stream), for
+ * the device that is current at the call: launches on different streams of one device may overlap, launches on one
+ * stream are ordered by the stream. Calls are serialised by one lock only while they enqueue. A buffer that has to grow
+ * is replaced and the old one freed by rf_gemm_destroy, so no call waits for the device (up to 32 streams per device
+ * have a buffer set of their own; a caller that cycles through more pays a device-wide wait when a set changes hands).
  */
 #ifndef RF_GEMM_H
 #define RF_GEMM_H

@@ -80,14 +80,30 @@ struct TunedPlan {
 
 // Buffers, counters and kernel attributes belong to a device: one State per device, chosen by the device that is
 // current at the call. Plans and the lock are shared by the process.
-struct State {
+//
+// Temporary device memory (split-K partial sums, stream-K slots and counters, staging copies of ragged operands) is
+// kept per (device, stream): two launches on different streams of one device never share a buffer, so they may overlap,
+// and launches on one stream are ordered by the stream. A buffer that has to grow is replaced, and the old one is kept
+// until rf_gemm_destroy: work enqueued earlier may still use it, and waiting for that work here would block the host
+// (and, with a timing callback of run() pending, deadlock against it).
+struct StreamBuffers {
+    hipStream_t stream = nullptr;
     uint8_t *pad = nullptr;              // staging for shapes the tiled kernels do not take as they are (see launch_padded)
     size_t pad_bytes = 0;
-    float *ws = nullptr;
+    float *ws = nullptr;                 // split-K partial sums / stream-K slots
     size_t ws_bytes = 0;
     unsigned *tile_count = nullptr;      // stream-K arrival counters, zero between launches
+    bool tile_count_zeroed = false;
+    uint64_t last_use = 0;
+};
+constexpr int kMaxStreamBuffers = 32;    // per device; one more stream takes over the least recently used set
+struct State {
+    std::vector<StreamBuffers> buffers;
+    std::vector<void *> retired;         // outgrown buffers, freed by rf_gemm_destroy
+    uint64_t tick = 0;
     bool attrs_set = false, grouped_attrs_set = false;
     int num_cu = 0;
+    std::mutex ev_mu;                    // guards free_events only: the timing callback takes no other lock
     std::vector<std::pair<hipEvent_t, hipEvent_t>> free_events;
 };
 struct Shared {
@@ -170,25 +186,94 @@ int ensure_device_info(State &s) {
     return RF_OK;
 }
 
-int ensure_workspace(State &s, size_t bytes) {
-    if (bytes <= s.ws_bytes) return RF_OK;
-    if (s.ws) {
-        RF_HIP(hipDeviceSynchronize());      // earlier launches may still read the old buffer
-        RF_HIP(hipFree(s.ws));
-        s.ws = nullptr;
-        s.ws_bytes = 0;
-    }
-    RF_HIP(hipMalloc((void **)&s.ws, bytes));
-    s.ws_bytes = bytes;
-    return RF_OK;
-}
-
 constexpr int kMaxStreamKTiles = 16384;
 
-int ensure_tile_counters(State &s) {
-    if (s.tile_count) return RF_OK;
-    RF_HIP(hipMalloc((void **)&s.tile_count, kMaxStreamKTiles * sizeof(unsigned)));
-    RF_HIP(hipMemset(s.tile_count, 0, kMaxStreamKTiles * sizeof(unsigned)));
+__global__ void zero_words(unsigned *p) { p[blockIdx.x * 256 + threadIdx.x] = 0u; }
+
+// hipMalloc that also works while the calling thread records a stream into a HIP graph: an allocation is not part
+// of the recorded work, so the capture mode is relaxed around it (under the default mode the call would fail and
+// invalidate the capture).
+hipError_t device_malloc(void **p, size_t bytes) {
+    hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+    hipError_t e = hipThreadExchangeStreamCaptureMode(&mode);
+    if (e != hipSuccess) return e;
+    e = hipMalloc(p, bytes);
+    (void)hipThreadExchangeStreamCaptureMode(&mode);
+    return e;
+}
+
+// Where a launch finds its temporary device memory: the growable buffers of its (device, stream).
+struct Mem {
+    State &s;
+    StreamBuffers *sb = nullptr;
+
+    template <typename T>
+    int grow(T *&buf, size_t &have, size_t need) {
+        if (need <= have) return RF_OK;
+        // the old buffer may still be read by launches enqueued earlier: keep it until rf_gemm_destroy
+        if (buf) s.retired.push_back(buf);
+        const size_t want = need > have + have / 2 ? need : have + have / 2;
+        buf = nullptr;
+        have = 0;
+        RF_HIP(device_malloc((void **)&buf, want));
+        have = want;
+        return RF_OK;
+    }
+    int pad(size_t bytes, uint8_t **out) {
+        int rc = grow(sb->pad, sb->pad_bytes, bytes);
+        *out = sb->pad;
+        return rc;
+    }
+    int workspace(size_t bytes, float **out) {
+        int rc = grow(sb->ws, sb->ws_bytes, bytes);
+        *out = sb->ws;
+        return rc;
+    }
+    int tile_counters(unsigned **out) {
+        if (!sb->tile_count) RF_HIP(device_malloc((void **)&sb->tile_count, kMaxStreamKTiles * sizeof(unsigned)));
+        if (!sb->tile_count_zeroed) {
+            // zeroed on the stream of the launch that follows (the kernels leave the counters at zero afterwards);
+            // a kernel and not a memset, so that the call may be recorded into a HIP graph. A recorded fill has not
+            // run yet, so it does not count: launches keep filling first until one has done so for real.
+            hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+            RF_HIP(hipStreamIsCapturing(sb->stream, &st));
+            hipLaunchKernelGGL(zero_words, dim3(kMaxStreamKTiles / 256), dim3(256), 0, sb->stream, sb->tile_count);
+            RF_HIP(hipGetLastError());
+            sb->tile_count_zeroed = st == hipStreamCaptureStatusNone;
+        }
+        *out = sb->tile_count;
+        return RF_OK;
+    }
+};
+
+// The buffer set of (current device, stream); the caller holds the lock. A set prepared by rf_gemm_init and not yet
+// bound to a stream is taken first. Past kMaxStreamBuffers streams the least recently used set changes hands, after
+// a device-wide wait (the only host wait in the launch path, and only for callers that cycle through that many streams).
+constexpr uintptr_t kUnboundStream = 1;  // not a valid stream handle
+int buffers_of(State &s, hipStream_t stream, StreamBuffers **out) {
+    StreamBuffers *unbound = nullptr, *lru = nullptr;
+    for (StreamBuffers &b : s.buffers) {
+        if (b.stream == stream) {
+            b.last_use = ++s.tick;
+            *out = &b;
+            return RF_OK;
+        }
+        if ((uintptr_t)b.stream == kUnboundStream) unbound = &b;
+        if (!lru || b.last_use < lru->last_use) lru = &b;
+    }
+    StreamBuffers *b = unbound;
+    if (!b && (int)s.buffers.size() < kMaxStreamBuffers) {
+        if (s.buffers.capacity() < (size_t)kMaxStreamBuffers) s.buffers.reserve(kMaxStreamBuffers);
+        s.buffers.emplace_back();
+        b = &s.buffers.back();
+    }
+    if (!b) {
+        RF_HIP(hipDeviceSynchronize());
+        b = lru;
+    }
+    b->stream = stream;
+    b->last_use = ++s.tick;
+    *out = b;
     return RF_OK;
 }
 
@@ -204,6 +289,13 @@ bool tiled_path_ok(const void *a, const void *b, const void *c, int m, int n) {
 
 bool persistent_ok(const Variant &v, int m, int n, int k) {
     return v.persistent && m % v.bm == 0 && n % v.bn == 0 && (k / rf::BK) % 2 == 0;
+}
+
+// Stream-K: at least one tile per workgroup (then a split tile has exactly two contributors, which is all the kernel
+// handles) and no more tiles than arrival counters.
+bool stream_k_ok(const Variant &v, int m, int n, int num_cu) {
+    const long t = (long)ceil_div(m, v.bm) * ceil_div(n, v.bn);
+    return v.streamk && t >= num_cu && t <= kMaxStreamKTiles;
 }
 
 // Plans measured on one MI355X by the tuner (python -m radeonflow_kernels_amd.tuner.gemm_tuner --all --emit).
@@ -227,7 +319,7 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
     auto usable = [&](const TunedPlan &p) {
         return p.m == m && p.n == n && p.k == k && p.variant < kNumVariants && p.split_k <= k / rf::BK &&
                (p.stream_k != RF_SCHEDULE_PERSISTENT || persistent_ok(kVariants[p.variant], m, n, k)) &&
-               (p.stream_k != RF_SCHEDULE_STREAM_K || kVariants[p.variant].streamk);
+               (p.stream_k != RF_SCHEDULE_STREAM_K || stream_k_ok(kVariants[p.variant], m, n, num_cu));
     };
     const TunedPlan *hit = nullptr;
     for (const TunedPlan &p : user_plans)
@@ -281,8 +373,8 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
 
 // The launch proper; the caller holds the lock and has checked shape and pointers. m_store >= 0: c has only m_store
 // (<= m) rows, the rest of the m rows of the operands are padding (one workgroup per tile schedules only).
-int launch_locked(State &s, const void *a, const void *b, const float *as, const float *bs, void *c, int m, int n, int k,
-                  const rf_gemm_config *user_cfg, hipStream_t stream, int m_store = -1) {
+int launch_locked(State &s, Mem &mem, const void *a, const void *b, const float *as, const float *bs, void *c, int m, int n,
+                  int k, const rf_gemm_config *user_cfg, hipStream_t stream, int m_store = -1) {
     int rc = RF_OK;
     if (m_store < 0) m_store = m;
     const bool tiled_ok = tiled_path_ok(a, b, c, m, n);
@@ -296,8 +388,7 @@ int launch_locked(State &s, const void *a, const void *b, const float *as, const
         if (cfg.stream_k == RF_SCHEDULE_STREAM_K) {
             const Variant &sv = kVariants[cfg.variant];
             if (!sv.streamk) return fail(RF_ERR_BAD_CONFIG, "this variant has no stream_k form");
-            const long t = (long)ceil_div(m, sv.bm) * ceil_div(n, sv.bn);
-            if (t < s.num_cu || t > kMaxStreamKTiles)
+            if (!stream_k_ok(sv, m, n, s.num_cu))
                 return fail(RF_ERR_BAD_CONFIG, "stream_k needs at least as many tiles as compute units");
         } else if (cfg.stream_k == RF_SCHEDULE_PERSISTENT) {
             if (!persistent_ok(kVariants[cfg.variant], m, n, k))
@@ -341,12 +432,14 @@ int launch_locked(State &s, const void *a, const void *b, const float *as, const
     }
     if (cfg.stream_k == RF_SCHEDULE_STREAM_K) {
         const int P = s.num_cu;
-        rc = ensure_tile_counters(s);
+        unsigned *tile_count = nullptr;
+        float *ws = nullptr;
+        rc = mem.tile_counters(&tile_count);
         if (rc != RF_OK) return rc;
-        rc = ensure_workspace(s, (size_t)2 * P * v.bm * v.bn * sizeof(float));
+        rc = mem.workspace((size_t)2 * P * v.bm * v.bn * sizeof(float), &ws);
         if (rc != RF_OK) return rc;
         hipLaunchKernelGGL(v.streamk, dim3(P), block, v.lds_bytes(), stream, (const uint8_t *)a, (const uint8_t *)b, as,
-                           bs, (uint16_t *)c, m, n, k, tiles_m, tiles_n, cfg.group_m, s.tile_count, s.ws);
+                           bs, (uint16_t *)c, m, n, k, tiles_m, tiles_n, cfg.group_m, tile_count, ws);
         RF_HIP(hipGetLastError());
         return RF_OK;
     }
@@ -356,14 +449,15 @@ int launch_locked(State &s, const void *a, const void *b, const float *as, const
         RF_HIP(hipGetLastError());
     } else {
         const size_t mn = (size_t)m * n;
-        rc = ensure_workspace(s, mn * splits * sizeof(float));
+        float *ws = nullptr;
+        rc = mem.workspace(mn * splits * sizeof(float), &ws);
         if (rc != RF_OK) return rc;
         hipLaunchKernelGGL(v.partial, grid, block, v.lds_bytes(), stream, (const uint8_t *)a, (const uint8_t *)b, as,
-                           bs, (void *)s.ws, m, n, k, kb_per_split, tiles_m, tiles_n, cfg.group_m, m);
+                           bs, (void *)ws, m, n, k, kb_per_split, tiles_m, tiles_n, cfg.group_m, m);
         RF_HIP(hipGetLastError());
         const size_t mn_store = (size_t)m_store * n;
         hipLaunchKernelGGL(rf::reduce_splitk_bf16, dim3((unsigned)((mn_store / 4 + 255) / 256)), dim3(256), 0, stream,
-                           (const float *)s.ws, (uint16_t *)c, mn_store, splits, mn);
+                           (const float *)ws, (uint16_t *)c, mn_store, splits, mn);
         RF_HIP(hipGetLastError());
     }
     return RF_OK;
@@ -377,19 +471,6 @@ int launch_locked(State &s, const void *a, const void *b, const float *as, const
 // nobody reads), the tiled kernels run on the padded shape under the automatic plan, and C is copied back without the
 // padding. b_scale needs no copy: ceil(N/128) does not change. The copies cost K*M (+ K*N when N is ragged) bytes.
 constexpr double kPadThresholdMacs = 2097152.0;            // below this the bounds-checked kernel is as fast
-
-int ensure_pad(State &s, size_t bytes) {
-    if (bytes <= s.pad_bytes) return RF_OK;
-    if (s.pad) {
-        RF_HIP(hipDeviceSynchronize());
-        RF_HIP(hipFree(s.pad));
-        s.pad = nullptr;
-        s.pad_bytes = 0;
-    }
-    RF_HIP(hipMalloc((void **)&s.pad, bytes));
-    s.pad_bytes = bytes;
-    return RF_OK;
-}
 
 // The grouped GEMM's staging copy: the caller's [rows][m_total] matrix (A with T = bytes, a_scale with T = float), in
 // which group g owns columns out_row_start[g] .. out_row_start[g+1]-1, is copied to [rows][m_pad] with group g starting
@@ -509,8 +590,8 @@ rf::GroupTable one_group(int cols, int cols_pad) {
     return t;
 }
 
-int launch_padded(State &s, const void *a, const void *b, const float *as, const float *bs, void *c, int m, int n, int k,
-                  hipStream_t stream) {
+int launch_padded(State &s, Mem &mem, const void *a, const void *b, const float *as, const float *bs, void *c, int m, int n,
+                  int k, hipStream_t stream) {
     auto pad16 = [](int x) { return x < 16 ? 16 : (x + 15) / 16 * 16; };
     auto align = [](size_t x) { return (x + 255) / 256 * 256; };
     const int mp = pad16(m), np = pad16(n), qk = k / rf::BK;
@@ -526,28 +607,29 @@ int launch_padded(State &s, const void *a, const void *b, const float *as, const
     const size_t off_b = off;  off += copy_b ? align((size_t)k * np) : 0;
     const size_t off_sa = off; off += copy_sa ? align((size_t)qk * mp * sizeof(float)) : 0;
     const size_t off_c = off;  off += copy_c ? align((size_t)mp * np * 2) : 0;
-    int rc = ensure_pad(s, off);
+    uint8_t *pad = nullptr;
+    int rc = mem.pad(off, &pad);
     if (rc != RF_OK) return rc;
     const void *a2 = a, *b2 = b;
     const float *as2 = as;
     void *c2 = c;
     if (copy_a && copy_sa) {
-        launch_pad_a_and_scales(a, as, m, mp, k, 1, s.pad + off_a, (float *)(s.pad + off_sa), one_group(m, mp), stream);
-        a2 = s.pad + off_a;
-        as2 = (const float *)(s.pad + off_sa);
+        launch_pad_a_and_scales(a, as, m, mp, k, 1, pad + off_a, (float *)(pad + off_sa), one_group(m, mp), stream);
+        a2 = pad + off_a;
+        as2 = (const float *)(pad + off_sa);
     } else if (copy_a) {                                   // M is fine, only the pointer is not aligned
         hipLaunchKernelGGL(pad_group_rows<uint8_t>, pad_grid(mp, 1, k), dim3(256), 0, stream, (const uint8_t *)a, m, mp, k, 1,
-                           s.pad + off_a, one_group(m, mp));
-        a2 = s.pad + off_a;
+                           pad + off_a, one_group(m, mp));
+        a2 = pad + off_a;
     }
     if (copy_b) {
         hipLaunchKernelGGL(pad_group_rows<uint8_t>, pad_grid(np, 1, k), dim3(256), 0, stream, (const uint8_t *)b, n, np, k, 1,
-                           s.pad + off_b, one_group(n, np));
-        b2 = s.pad + off_b;
+                           pad + off_b, one_group(n, np));
+        b2 = pad + off_b;
     }
-    if (copy_c) c2 = s.pad + off_c;
+    if (copy_c) c2 = pad + off_c;
     RF_HIP(hipGetLastError());
-    rc = launch_locked(s, a2, b2, as2, bs, c2, mp, np, k, &cfg, stream, copy_c ? mp : m);
+    rc = launch_locked(s, mem, a2, b2, as2, bs, c2, mp, np, k, &cfg, stream, copy_c ? mp : m);
     if (rc != RF_OK) return rc;
     if (copy_c)
         RF_HIP(hipMemcpy2DAsync(c, (size_t)n * 2, c2, (size_t)np * 2, (size_t)n * 2, m, hipMemcpyDeviceToDevice, stream));
@@ -565,9 +647,12 @@ int launch(const void *a, const void *b, const float *as, const float *bs, void 
     std::lock_guard<std::mutex> lock(shared().mu);
     int rc = ensure_device_info(s);
     if (rc != RF_OK) return rc;
+    Mem mem{s};
+    rc = buffers_of(s, stream, &mem.sb);
+    if (rc != RF_OK) return rc;
     if (!user_cfg && !tiled_path_ok(a, b, c, m, n) && (double)m * n * k >= kPadThresholdMacs)
-        return launch_padded(s, a, b, as, bs, c, m, n, k, stream);
-    return launch_locked(s, a, b, as, bs, c, m, n, k, user_cfg, stream);
+        return launch_padded(s, mem, a, b, as, bs, c, m, n, k, stream);
+    return launch_locked(s, mem, a, b, as, bs, c, m, n, k, user_cfg, stream);
 }
 
 // ---- timing record for run() ----------------------------------------------------------------
@@ -588,7 +673,9 @@ void timer_callback(hipStream_t, hipError_t status, void *user) {
     }
     State &s = *job->owner;               // the callback thread has no current device of its own
     {
-        std::lock_guard<std::mutex> lock(shared().mu);
+        // the pool has a lock of its own: the launch path may hold the library lock while it waits for the device,
+        // and the device may be waiting for this callback
+        std::lock_guard<std::mutex> lock(s.ev_mu);
         s.free_events.emplace_back(job->start, job->stop);   // recycled, unlike the reference's growing list
     }
     delete job;
@@ -715,23 +802,29 @@ int rf_gemm_init(size_t workspace_bytes) {
     std::lock_guard<std::mutex> lock(shared().mu);
     int rc = ensure_device_info(s);
     if (rc != RF_OK) return rc;
-    return ensure_workspace(s, workspace_bytes);
+    if (workspace_bytes == 0) return RF_OK;
+    // a buffer set that belongs to no stream yet: the first stream that needs one takes it over
+    StreamBuffers *sb = nullptr;
+    rc = buffers_of(s, (hipStream_t)kUnboundStream, &sb);
+    if (rc != RF_OK) return rc;
+    Mem mem{s, sb};
+    float *ws = nullptr;
+    return mem.workspace(workspace_bytes, &ws);
 }
 
 void rf_gemm_destroy(void) {
     State &s = state();
     std::lock_guard<std::mutex> lock(shared().mu);
-    if (s.ws) {
-        (void)hipDeviceSynchronize();
-        (void)hipFree(s.ws);
+    if (!s.buffers.empty() || !s.retired.empty()) (void)hipDeviceSynchronize();   // launches may still use them
+    for (StreamBuffers &b : s.buffers) {
+        if (b.ws) (void)hipFree(b.ws);
+        if (b.pad) (void)hipFree(b.pad);
+        if (b.tile_count) (void)hipFree(b.tile_count);
     }
-    s.ws = nullptr;
-    s.ws_bytes = 0;
-    if (s.tile_count) (void)hipFree(s.tile_count);
-    s.tile_count = nullptr;
-    if (s.pad) (void)hipFree(s.pad);
-    s.pad = nullptr;
-    s.pad_bytes = 0;
+    s.buffers.clear();
+    for (void *p : s.retired) (void)hipFree(p);
+    s.retired.clear();
+    std::lock_guard<std::mutex> ev_lock(s.ev_mu);
     for (auto &p : s.free_events) {
         (void)hipEventDestroy(p.first);
         (void)hipEventDestroy(p.second);
@@ -858,24 +951,32 @@ int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const flo
         for (int g = 0; g <= rf::kMaxGroups; g++) table.out_row_start[g] = row_offsets[g < groups ? g : groups];
         m_rows = at;
         const size_t a_bytes = ((size_t)k * m_rows + 255) / 256 * 256;
-        rc = ensure_pad(s, a_bytes + (size_t)qk * m_rows * sizeof(float));
+        StreamBuffers *sb = nullptr;
+        rc = buffers_of(s, stream, &sb);
         if (rc != RF_OK) return rc;
-        launch_pad_a_and_scales(a, as, m_total, m_rows, k, groups, s.pad, (float *)(s.pad + a_bytes), table, stream);
+        Mem mem{s, sb};
+        uint8_t *pad = nullptr;
+        rc = mem.pad(a_bytes + (size_t)qk * m_rows * sizeof(float), &pad);
+        if (rc != RF_OK) return rc;
+        launch_pad_a_and_scales(a, as, m_total, m_rows, k, groups, pad, (float *)(pad + a_bytes), table, stream);
         RF_HIP(hipGetLastError());
-        a = s.pad;
-        as = (const float *)(s.pad + a_bytes);
+        a = pad;
+        as = (const float *)(pad + a_bytes);
     } else {
         for (int g = 0; g <= rf::kMaxGroups; g++)
             table.row_start[g] = table.out_row_start[g] = row_offsets[g < groups ? g : groups];
     }
     if (variant < 0) {
         // the largest tile that still gives every CU a workgroup; failing that, the one with the most workgroups
-        variant = kNumGroupedVariants - 1;
-        for (int v = 0; v < kNumGroupedVariants; v++)
-            if (grouped_tiles(kGroupedVariants[v], row_offsets, groups, n) >= s.num_cu) {
-                variant = v;
-                break;
-            }
+        variant = -1;
+        long most = -1;
+        int most_v = 0;
+        for (int v = 0; v < kNumGroupedVariants && variant < 0; v++) {
+            const long t = grouped_tiles(kGroupedVariants[v], row_offsets, groups, n);
+            if (t >= s.num_cu) variant = v;
+            if (t > most) { most = t; most_v = v; }
+        }
+        if (variant < 0) variant = most_v;
         // Every row tile of a group streams the group's whole weight block, and with small groups that traffic is the
         // bound. 128-row tiles are the better choice exactly when they do not add row tiles (nearly all groups have at
         // most 128 rows): same weight traffic, half the padding. Measured, N=4096 K=7168: 32 groups of 16..128 rows
@@ -938,7 +1039,7 @@ void run(void *a, void *b, void *as, void *bs, void *c, int m, int n, int k, Per
         State &s = state();
         job->owner = &s;
         {
-            std::lock_guard<std::mutex> lock(shared().mu);
+            std::lock_guard<std::mutex> lock(s.ev_mu);
             if (!s.free_events.empty()) {
                 job->start = s.free_events.back().first;
                 job->stop = s.free_events.back().second;

@@ -65,23 +65,23 @@ __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __builtin
 // Maximum over each aligned group of 16 lanes, left in all of them, for N unsigned values at once: four DPP steps
 // (swap within pairs, within quads, rotate the 16-lane row by 4 and by 8) instead of LDS-crossbar shuffles, each one
 // v_max_u32 with a DPP operand. Written as asm because the compiler emits move + max for the builtin form. A DPP
-// operand must not be read within two instructions of the VALU write that produced it: the first step carries its
-// own wait, later steps of one value are N >= 3 volatile statements apart.
+// operand must not be read within two instructions of the VALU write that produced it, and the compiler's hazard
+// recogniser does not look inside asm statements (it may also place a register copy right in front of one): every
+// step carries its own two wait states.
 template <int N>
 __device__ __forceinline__ void max_over_16_lanes(uint32_t (&a)[N]) {
-    static_assert(N >= 3, "steps of one value must be at least two instructions apart");
 #pragma unroll
     for (int i = 0; i < N; i++)
         asm volatile("s_nop 1\n\tv_max_u32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf" : "+v"(a[i]));
 #pragma unroll
     for (int i = 0; i < N; i++)
-        asm volatile("v_max_u32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf" : "+v"(a[i]));
+        asm volatile("s_nop 1\n\tv_max_u32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf" : "+v"(a[i]));
 #pragma unroll
     for (int i = 0; i < N; i++)
-        asm volatile("v_max_u32_dpp %0, %0, %0 row_ror:4 row_mask:0xf bank_mask:0xf" : "+v"(a[i]));
+        asm volatile("s_nop 1\n\tv_max_u32_dpp %0, %0, %0 row_ror:4 row_mask:0xf bank_mask:0xf" : "+v"(a[i]));
 #pragma unroll
     for (int i = 0; i < N; i++)
-        asm volatile("v_max_u32_dpp %0, %0, %0 row_ror:8 row_mask:0xf bank_mask:0xf" : "+v"(a[i]));
+        asm volatile("s_nop 1\n\tv_max_u32_dpp %0, %0, %0 row_ror:8 row_mask:0xf bank_mask:0xf" : "+v"(a[i]));
     asm volatile("s_nop 1" ::: "memory");     // the compiler may follow up with a DPP or lane-crossing read of a[N-1]
 }
 

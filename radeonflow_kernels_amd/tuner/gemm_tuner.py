@@ -98,13 +98,23 @@ def tune_shape(rfk, m, n, k, log=print):
     return out
 
 
+def best_for_table(cands):
+    """The winner that goes into a plan table or plan file: the fastest candidate that is not a stream-K plan. Whether
+    stream-K can run depends on the compute-unit count of the device (it needs at least one tile per unit), so a table
+    that may be read on another device does not carry it; it stays available through an explicit rf_gemm_config."""
+    for c in cands:
+        if c["stream_k"] != 1:
+            return c
+    return None
+
+
 def emit_plans(results, path=PLANS_INC):
     lines = ["// Generated by radeonflow_kernels_amd/tuner/gemm_tuner.py --all [--extended] --emit on one MI355X; do not edit by hand.",
              "// {M, N, K, variant, split_k, group_m, stream_k},   best time, TFLOP/s"]
     for (m, n, k), cands in results.items():
-        if not cands:
+        b = best_for_table(cands)
+        if b is None:
             continue
-        b = cands[0]
         lines.append("{%d, %d, %d, %d, %d, %d, %d},   // %.2f us, %.1f TFLOP/s" % (
             m, n, k, b["variant"], b["split_k"], b["group_m"], b["stream_k"], b["us"], b["tflops"]))
     with open(path, "w") as f:
@@ -148,8 +158,8 @@ def main():
     if a.emit_file:
         with open(a.emit_file, "a") as f:
             for (m, n, k), cands in results.items():
-                if cands:
-                    b = cands[0]
+                b = best_for_table(cands)
+                if b is not None:
                     f.write("%d %d %d %d %d %d %d   # %.2f us, %.1f TFLOP/s\n" % (
                         m, n, k, b["variant"], b["split_k"], b["group_m"], b["stream_k"], b["us"], b["tflops"]))
         print("appended to", a.emit_file)

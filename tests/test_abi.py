@@ -150,3 +150,16 @@ def test_compiled_in_plan_table_only_holds_plans_its_shapes_can_run():
         if schedule == 2:
             assert L.rf_gemm_variant_has_persistent(variant) == 1 and split == 1
             assert m % bm.value == 0 and n % bn.value == 0 and (k // 128) % 2 == 0
+
+
+def test_tuner_never_writes_a_stream_k_winner_into_a_table_or_plan_file(tmp_path):
+    """Stream-K needs one tile per compute unit of the device it runs on, so tables and plan files carry the fastest
+    plan of another schedule instead."""
+    from radeonflow_kernels_amd.tuner import gemm_tuner as t
+    cand = lambda sk, us: dict(variant=0, split_k=1, group_m=4, stream_k=sk, us=us, tflops=1.0)
+    assert t.best_for_table([cand(1, 10.0), cand(2, 11.0), cand(0, 12.0)])["stream_k"] == 2
+    assert t.best_for_table([cand(1, 10.0)]) is None and t.best_for_table([]) is None
+    out = tmp_path / "plans.inc"
+    t.emit_plans({(512, 512, 256): [cand(1, 10.0), cand(0, 12.0)], (256, 256, 256): [cand(1, 9.0)]}, str(out))
+    lines = [l for l in out.read_text().splitlines() if l.startswith("{")]
+    assert len(lines) == 1 and lines[0].startswith("{512, 512, 256, 0, 1, 4, 0}")
