@@ -75,6 +75,19 @@ void run(void *a, void *b, void *as, void *bs, void *c, int m, int n, int k, Per
 int rf_fp8_gemm(const void *a, const void *b, const float *as, const float *bs, void *c,
                 int m, int n, int k, hipStream_t stream);
 
+/* rf_fp8_gemm for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc. No counterpart in the reference (its launcher allocates a fixed workspace with
+ * hipMalloc on first use, src/gemm/gemm_launcher.cpp:30-36). Same arguments, plan choice and result bits as
+ * rf_fp8_gemm, but split-K partial sums and the staging copies of ragged or unaligned operands live in a static
+ * device array of rf_gemm_static_scratch_bytes() bytes (32 MiB; every GPU the library has run on holds one until the
+ * process ends), and the call allocates and frees nothing. A shape whose plan needs more scratch memory than that
+ * fails with RF_ERR_BAD_CONFIG (rf_gemm_last_error() gives the bytes needed), as does a stream-K plan from a plan
+ * file. All calls on one GPU share that GPU's array: two calls that overlap in time (different streams, or graph
+ * replays beside eager launches) race; calls on one stream are ordered by the stream. */
+int rf_fp8_gemm_static(const void *a, const void *b, const float *as, const float *bs, void *c,
+                       int m, int n, int k, hipStream_t stream);
+size_t rf_gemm_static_scratch_bytes(void);
+
 /* As rf_fp8_gemm with an explicit plan (cfg == NULL selects automatically). This is what the tuner
  * drives instead of recompiling a template per configuration (tuner/template/gemm_perf.cpp:21-38). */
 int rf_fp8_gemm_ex(const void *a, const void *b, const float *as, const float *bs, void *c,

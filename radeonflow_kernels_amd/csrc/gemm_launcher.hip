@@ -18,6 +18,12 @@
 #include "fp8_gemm_persistent.h"
 #include "quantize_kernels.h"
 
+// Scratch memory of rf_fp8_gemm_static, the entry point that allocates nothing: split-K partial sums and staging
+// copies live here instead of in buffers from hipMalloc. Every device the library runs on holds its own copy at its
+// own address until the process ends; host code never uses this name as an address (see ensure_device_info).
+constexpr size_t kStaticScratchBytes = (size_t)32 << 20;
+static __device__ __align__(256) uint8_t scratch[kStaticScratchBytes];
+
 namespace {
 
 thread_local std::string g_last_error;
@@ -103,6 +109,7 @@ struct State {
     uint64_t tick = 0;
     bool attrs_set = false, grouped_attrs_set = false;
     int num_cu = 0;
+    uint8_t *static_scratch = nullptr;   // this device's copy of the file-scope scratch array (rf_fp8_gemm_static)
     std::mutex ev_mu;                    // guards free_events only: the timing callback takes no other lock
     std::vector<std::pair<hipEvent_t, hipEvent_t>> free_events;
 };
@@ -182,6 +189,10 @@ int ensure_device_info(State &s) {
             RF_HIP(hipFuncSetAttribute((const void *)v.persistent, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        v.lds_persistent));
     }
+    // the device address of this device's copy of the scratch array (the array's name is only a host-side handle)
+    void *scratch_ptr = nullptr;
+    RF_HIP(hipGetSymbolAddress(&scratch_ptr, HIP_SYMBOL(scratch)));
+    s.static_scratch = (uint8_t *)scratch_ptr;
     s.attrs_set = true;
     return RF_OK;
 }
@@ -202,10 +213,14 @@ hipError_t device_malloc(void **p, size_t bytes) {
     return e;
 }
 
-// Where a launch finds its temporary device memory: the growable buffers of its (device, stream).
+// Where a launch finds its temporary device memory: the growable buffers of its (device, stream), or, for
+// rf_fp8_gemm_static, consecutive pieces of the device's static scratch array (nothing is allocated; a launch that
+// needs more than the array holds fails).
 struct Mem {
     State &s;
-    StreamBuffers *sb = nullptr;
+    StreamBuffers *sb = nullptr;         // growable buffers (null in static mode)
+    uint8_t *fixed = nullptr;            // static mode: this device's scratch array
+    size_t fixed_used = 0;
 
     template <typename T>
     int grow(T *&buf, size_t &have, size_t need) {
@@ -219,17 +234,30 @@ struct Mem {
         have = want;
         return RF_OK;
     }
+    int take_fixed(size_t bytes, void **out, const char *what) {
+        const size_t at = (fixed_used + 255) / 256 * 256;
+        if (at + bytes > kStaticScratchBytes)
+            return fail(RF_ERR_BAD_CONFIG, std::string("rf_fp8_gemm_static: this shape needs ") + std::to_string(at + bytes) +
+                                               " bytes of scratch memory (" + what + "), the static array holds " +
+                                               std::to_string(kStaticScratchBytes));
+        *out = fixed + at;
+        fixed_used = at + bytes;
+        return RF_OK;
+    }
     int pad(size_t bytes, uint8_t **out) {
+        if (fixed) return take_fixed(bytes, (void **)out, "staging copy of ragged or unaligned operands");
         int rc = grow(sb->pad, sb->pad_bytes, bytes);
         *out = sb->pad;
         return rc;
     }
     int workspace(size_t bytes, float **out) {
+        if (fixed) return take_fixed(bytes, (void **)out, "split-K partial sums");
         int rc = grow(sb->ws, sb->ws_bytes, bytes);
         *out = sb->ws;
         return rc;
     }
     int tile_counters(unsigned **out) {
+        if (fixed) return fail(RF_ERR_BAD_CONFIG, "rf_fp8_gemm_static: the stream-K schedule is not available");
         if (!sb->tile_count) RF_HIP(device_malloc((void **)&sb->tile_count, kMaxStreamKTiles * sizeof(unsigned)));
         if (!sb->tile_count_zeroed) {
             // zeroed on the stream of the launch that follows (the kernels leave the counters at zero afterwards);
@@ -637,7 +665,7 @@ int launch_padded(State &s, Mem &mem, const void *a, const void *b, const float 
 }
 
 int launch(const void *a, const void *b, const float *as, const float *bs, void *c, int m, int n, int k,
-           const rf_gemm_config *user_cfg, hipStream_t stream) {
+           const rf_gemm_config *user_cfg, hipStream_t stream, bool static_memory = false) {
     g_last_error.clear();
     if (m < 1 || n < 1 || k < rf::BK || k % rf::BK != 0)
         return fail(RF_ERR_BAD_SHAPE, "unsupported shape M=" + std::to_string(m) + " N=" + std::to_string(n) +
@@ -648,8 +676,12 @@ int launch(const void *a, const void *b, const float *as, const float *bs, void 
     int rc = ensure_device_info(s);
     if (rc != RF_OK) return rc;
     Mem mem{s};
-    rc = buffers_of(s, stream, &mem.sb);
-    if (rc != RF_OK) return rc;
+    if (static_memory) {
+        mem.fixed = s.static_scratch;
+    } else {
+        rc = buffers_of(s, stream, &mem.sb);
+        if (rc != RF_OK) return rc;
+    }
     if (!user_cfg && !tiled_path_ok(a, b, c, m, n) && (double)m * n * k >= kPadThresholdMacs)
         return launch_padded(s, mem, a, b, as, bs, c, m, n, k, stream);
     return launch_locked(s, mem, a, b, as, bs, c, m, n, k, user_cfg, stream);
@@ -689,6 +721,13 @@ int rf_fp8_gemm(const void *a, const void *b, const float *as, const float *bs, 
                 hipStream_t stream) {
     return launch(a, b, as, bs, c, m, n, k, nullptr, stream);
 }
+
+int rf_fp8_gemm_static(const void *a, const void *b, const float *as, const float *bs, void *c, int m, int n, int k,
+                       hipStream_t stream) {
+    return launch(a, b, as, bs, c, m, n, k, nullptr, stream, /*static_memory=*/true);
+}
+
+size_t rf_gemm_static_scratch_bytes(void) { return kStaticScratchBytes; }
 
 int rf_fp8_gemm_ex(const void *a, const void *b, const float *as, const float *bs, void *c, int m, int n, int k,
                    const rf_gemm_config *cfg, hipStream_t stream) {

@@ -40,7 +40,8 @@ class PerfMetrics(ctypes.Structure):
 EXPORTS = ("run", "rf_fp8_gemm", "rf_fp8_gemm_ex", "rf_gemm_select_config", "rf_gemm_num_variants",
            "rf_gemm_variant_info", "rf_gemm_variant_has_stream_k", "rf_gemm_variant_has_persistent", "rf_gemm_workspace_bytes", "rf_gemm_init", "rf_gemm_destroy",
            "rf_gemm_last_error", "rf_fp8_gemm_grouped", "rf_quantize_a_f32", "rf_quantize_a_bf16", "rf_quantize_b_f32", "rf_quantize_b_bf16",
-           "rf_cast_f32_to_e4m3fn", "rf_gemm_load_plans", "rf_gemm_clear_plans", "rf_fp8_gemm_time")
+           "rf_cast_f32_to_e4m3fn", "rf_gemm_load_plans", "rf_gemm_clear_plans", "rf_fp8_gemm_time", "rf_fp8_gemm_static",
+           "rf_gemm_static_scratch_bytes")
 
 
 def lib():
@@ -56,6 +57,10 @@ def lib():
         L.run.restype = None
         L.rf_fp8_gemm.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, vp]
         L.rf_fp8_gemm.restype = i32
+        L.rf_fp8_gemm_static.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, vp]
+        L.rf_fp8_gemm_static.restype = i32
+        L.rf_gemm_static_scratch_bytes.argtypes = []
+        L.rf_gemm_static_scratch_bytes.restype = ctypes.c_size_t
         L.rf_fp8_gemm_ex.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, ctypes.POINTER(GemmConfig), vp]
         L.rf_fp8_gemm_ex.restype = i32
         L.rf_fp8_gemm_time.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, ctypes.POINTER(GemmConfig), i32, i32,
@@ -127,6 +132,18 @@ def fp8_mm(a, b, a_scale, b_scale, c, config=None):
                               m, n, k, cfg, stream)
     if rc != RF_OK:
         raise RuntimeError("rf_fp8_gemm failed (%d): %s" % (rc, last_error()))
+
+
+def fp8_mm_static(a, b, a_scale, b_scale, c):
+    """fp8_mm through rf_fp8_gemm_static: same result, no device memory is allocated or freed by the call (temporary
+    data lives in a static 32 MiB device array; shapes that need more raise)."""
+    m, n, k = _check_layout(a, b, a_scale, b_scale, c)
+    stream = ctypes.c_void_p(torch.cuda.current_stream(a.device).cuda_stream)
+    with torch.cuda.device(a.device):
+        rc = lib().rf_fp8_gemm_static(a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(), c.data_ptr(),
+                                      m, n, k, stream)
+    if rc != RF_OK:
+        raise RuntimeError("rf_fp8_gemm_static failed (%d): %s" % (rc, last_error()))
 
 
 def fp8_mm_time(a, b, a_scale, b_scale, c, config=None, warmup=3, iters=20):
