@@ -1,16 +1,24 @@
 #!/usr/bin/env python3
 """Benchmark of the FP8 blockwise-scaled GEMM on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config C2] [--all] [--no-cpu]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config Cx] [--all] [--no-cpu]
 
 A step is one GEMM of the headline shape (M=6144, N=4608, K=7168) on synthetic inputs that are
 already resident in HBM (seeded N(0,1) fp32, quantised to e4m3fn with amax/448 block scales).
-`value` comes from K back-to-back launches between two HIP events on the launch stream; the line
-also carries the min / median of individually timed launches, a run with operands rotated out of the
-Infinity Cache, the roofline fraction, the CPU baseline and the correctness gate against the oracle.
-Prints ONE JSON line on stdout; the per-config table (with --all: time + correctness gate for all
-five configurations) goes to stderr.
+`value` comes from K back-to-back launches between two HIP events on the launch stream, issued by
+the library's own launch loop with no host gap after a clock-settling phase (`settle_launches`, about
+0.4 s of the same launch, whatever --warmup says: the shader clock and the board power need tens of
+milliseconds of load to reach their steady state) and W warm-up launches. The first K launches of
+the process after only W warm-up launches are reported beside it (`cold_clock_burst`). The line also
+carries the min / median of individually timed launches, a run with operands rotated out of the
+Infinity Cache, the roofline fraction, the CPU baseline, the correctness gate against the oracle and,
+without --config, `all_configs`: time, roofline fraction and correctness gate of all five
+configurations. With --config Cx only that configuration is run (this is the form the rocprofv3
+summaries under profiles/ are taken with). --all adds quantisers, the grouped form, operand-bit
+variations and the register-only MFMA ceiling. Prints ONE JSON line on stdout; tables go to stderr.
 """
+import glob
+import hashlib
 import argparse
 import json
 import os
@@ -34,8 +42,45 @@ CONFIGS = {
     "C5": (1024, 576, 7168, 12346),
 }
 RTOL, ATOL, ATOL_REFERENCE = 2e-2, 1e-2, 1e-3
-TRAFFIC_C2_BYTES = 394.2e6
-TRAFFIC_C2_NOTE = "fetch 337.6 MB + write 56.6 MB per launch, profiles/gemm_fp8_blockscale_persistent_C2_hbm_traffic.txt"
+SETTLE_SECONDS = 0.4
+KERNEL_SOURCES = ("fp8_gemm_kernels.h", "fp8_gemm_persistent.h")
+
+
+def kernel_source_sha():
+    """Short hash of the GEMM kernel sources: a traffic figure in profiles/ belongs to the kernels it was measured on."""
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "radeonflow_kernels_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:12]
+
+
+def measured_traffic(config, cfg):
+    """HBM-side bytes per launch from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summaries under profiles/ (lines
+    '@traffic config=C2 plan=0,1,2 fetch_kib=... write_kib=... fetch_factor=... write_factor=... source_sha=...').
+    Returns (bytes, note), or (None, why) when there is no summary for this configuration and plan or when the kernel
+    sources have changed since it was taken."""
+    plan = "%d,%d,%d" % (cfg.variant, cfg.split_k, cfg.stream_k)
+    why = "no rocprofv3 traffic summary for %s under profiles/" % config
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*hbm_traffic*.txt"))):
+        for line in open(path):
+            if not line.startswith("@traffic"):
+                continue
+            kv = dict(x.split("=", 1) for x in line.split()[1:])
+            if kv.get("config") != config:
+                continue
+            if kv.get("plan") != plan:
+                why = "%s was taken with plan %s, this run uses %s" % (os.path.basename(path), kv.get("plan"), plan)
+                continue
+            if kv.get("source_sha") != kernel_source_sha():
+                why = "%s was taken on other kernel sources (%s, now %s)" % (os.path.basename(path), kv.get("source_sha"),
+                                                                            kernel_source_sha())
+                continue
+            fetch = float(kv["fetch_kib"]) * float(kv["fetch_factor"]) * 1024
+            write = float(kv["write_kib"]) * float(kv["write_factor"]) * 1024
+            return fetch + write, "fetch %.1f MB + write %.1f MB per launch, profiles/%s" % (
+                fetch / 1e6, write / 1e6, os.path.basename(path))
+    return None, why
 
 
 def algorithmic_bytes(m, n, k):
@@ -51,8 +96,21 @@ def to_gpu(data):
     return colmajor(a), colmajor(b), colmajor(sa), colmajor(sb), torch.zeros(c.shape, dtype=torch.bfloat16, device="cuda")
 
 
+def settled_us(rfk, g, steps, warmup, settle_seconds=SETTLE_SECONDS):
+    """Average microseconds per GEMM over `steps` launches, after a settling phase of about `settle_seconds` of the same
+    launch plus `warmup` launches. Everything is enqueued back to back by one call of the library's launch loop
+    (rf_fp8_gemm_time: HIP events on the launch stream around the last `steps` launches), so there is no host gap
+    between settling and timing. Returns (us, settle_launches)."""
+    est = rfk.fp8_mm_time(*g, warmup=1, iters=3)
+    settle = max(1, int(settle_seconds * 1e6 / max(est, 1.0)))
+    torch.cuda.synchronize()
+    us = rfk.fp8_mm_time(*g, warmup=settle + warmup, iters=steps)
+    torch.cuda.synchronize()
+    return us, settle
+
+
 def time_gemm(rfk, sets, steps, warmup, stream):
-    """Average microseconds per GEMM over `steps` back-to-back launches, HIP events on the launch stream.
+    """Average microseconds per GEMM over `steps` back-to-back launches from Python, HIP events on the launch stream.
     `sets` is a list of operand tuples used in rotation (one tuple: operands stay warm in L2 / Infinity Cache)."""
     with torch.cuda.stream(stream):
         for i in range(warmup):
@@ -68,6 +126,18 @@ def time_gemm(rfk, sets, steps, warmup, stream):
         stream.synchronize()
         torch.cuda.synchronize()
     return e0.elapsed_time(e1) * 1e3 / steps
+
+
+def roofline_of(m, n, k, us):
+    """The roofline that bounds the shape (the larger of flop / fp8 peak and algorithmic bytes / HBM peak) and the
+    fraction of it a launch of `us` microseconds reaches."""
+    flop, nbytes = 2.0 * m * n * k, algorithmic_bytes(m, n, k)
+    tflops, gbs = flop / us / 1e6, nbytes / us / 1e3
+    if flop / (PEAK_FP8_TFLOPS * 1e12) >= nbytes / (PEAK_HBM_GBS * 1e9):
+        return {"bound": "mfma", "achieved": round(tflops, 2), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(tflops / PEAK_FP8_TFLOPS, 4)}
+    return {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "frac": round(gbs / PEAK_HBM_GBS, 4)}
 
 
 def clock_under_load(rfk, g, seconds, us_per_launch):
@@ -158,15 +228,60 @@ def parity_report(rfk, cref, rk, data, g, stream, expect=None, truth_rows=64):
             "elements": int(m * n), "pass": bad == 0}
 
 
+def measure_config(rfk, cref, rk, name, steps, warmup, stream, with_cpu, settle_seconds, keep=False):
+    """One configuration: inputs, settled launch time, roofline fraction, correctness gate. Returns the record (and
+    the inputs with keep=True)."""
+    m, n, k, seed = CONFIGS[name]
+    t0 = time.time()
+    data = rk.generate_input_blockquant(m, n, k, seed)
+    g = to_gpu(data)
+    gen_s = time.time() - t0
+    cold = rfk.fp8_mm_time(*g, warmup=warmup, iters=steps) if keep else None     # the process's first launches
+    us, settle = settled_us(rfk, g, steps, warmup, settle_seconds)
+    cfg = rfk.select_config(m, n, k)
+    schedule = {0: "gemm_fp8_blockscale_tile", 1: "gemm_fp8_blockscale_streamk", 2: "gemm_fp8_blockscale_persistent"}
+    launches = 1 if cfg.split_k == 1 else 2
+    rec = {"shape": [m, n, k], "us_per_gemm": round(us, 2), "settle_launches": settle,
+           "tflops": round(2.0 * m * n * k / us / 1e6, 1), "gbs_algorithmic": round(algorithmic_bytes(m, n, k) / us / 1e3, 1),
+           "roofline": roofline_of(m, n, k, us),
+           "plan": {"variant": cfg.variant, "split_k": cfg.split_k, "group_m": cfg.group_m, "stream_k": cfg.stream_k},
+           "kernel": "%s (variant %d, split_k %d)%s" % (schedule.get(cfg.stream_k, "?"), cfg.variant, cfg.split_k,
+                                                         " + reduce_splitk_bf16" if launches == 2 else ""),
+           "kernel_launches_per_gemm": launches}
+    traffic, note = measured_traffic(name, cfg)
+    rec["roofline"]["traffic"] = traffic
+    rec["roofline"]["traffic_note"] = note
+    expect = cpu_s = None
+    if with_cpu:
+        a, b, sa, sb, c = data
+        if keep:
+            # CPU baseline = the oracle's torch restatement of the reference path (dequantise, fp32 matmul, bf16) on
+            # the host cores, whole workload, best of 3 after a small warm-up
+            rk.ref_kernel((a[:128], b, sa[:128], sb, torch.zeros((128, n), dtype=torch.bfloat16)))
+            cpu_s = float("inf")
+            for _ in range(3):
+                t0 = time.perf_counter()
+                expect = rk.ref_kernel((a, b, sa, sb, torch.zeros((m, n), dtype=torch.bfloat16)))
+                cpu_s = min(cpu_s, time.perf_counter() - t0)
+        par = parity_report(rfk, cref, rk, data, g, stream, expect)
+        rec["parity"] = par if keep else {"mismatches": par["mismatches"],
+                                          "mismatches_at_reference_atol_1e-3": par["mismatches_at_reference_atol_1e-3"],
+                                          "max_abs_err": par["max_abs_err"], "elements": par["elements"], "pass": par["pass"]}
+    if keep:
+        return rec, data, g, gen_s, cold, cpu_s
+    return rec
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=200,
-                    help="untimed launches first; the GPU clock needs tens of milliseconds of load to settle")
-    ap.add_argument("--config", default="C2", choices=sorted(CONFIGS))
-    ap.add_argument("--all", action="store_true", help="also time the other four configurations (stderr table)")
+    ap.add_argument("--warmup", type=int, default=200, help="untimed launches directly before the timed ones")
+    ap.add_argument("--config", default=None, choices=sorted(CONFIGS),
+                    help="run only this configuration (default: C2 as the headline plus all_configs)")
+    ap.add_argument("--all", action="store_true", help="also quantisers, grouped form, operand bits, MFMA ceiling")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity gate")
+    ap.add_argument("--settle", type=float, default=SETTLE_SECONDS, help="seconds of launches before the timed region")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (output tiles are independent: "
@@ -185,38 +300,24 @@ def main():
     derived_peak = prop.multi_processor_count * clock_mhz * 1e6 * 8192 / 1e12
     stream = torch.cuda.Stream()
 
-    m, n, k, seed = CONFIGS[args.config]
-    t0 = time.time()
-    data = rk.generate_input_blockquant(m, n, k, seed)
-    g = to_gpu(data)
-    gen_s = time.time() - t0
-
-    us = time_gemm(rfk, [g], args.steps, args.warmup, stream)
+    headline = args.config or "C2"
+    m, n, k, seed = CONFIGS[headline]
+    rec, data, g, gen_s, us_burst, cpu_s = measure_config(rfk, cref, rk, headline, args.steps, args.warmup, stream,
+                                                          not args.no_cpu, args.settle, keep=True)
+    us = rec["us_per_gemm"]
+    flop = 2.0 * m * n * k
+    tflops = flop / us / 1e6
+    with torch.cuda.stream(stream):
+        rfk.fp8_mm_time(*g, warmup=rec["settle_launches"] // 2, iters=1)      # the clock falls back within milliseconds
     samples = sorted(per_launch_us(rfk, g, max(20, min(args.steps, 200)), stream))
     # operands that are not in the 256 MB Infinity Cache: rotate enough copies that a set is evicted before its turn
     set_bytes = algorithmic_bytes(m, n, k)
     ncopies = max(3, int(2 * 256e6 / set_bytes) + 1)
     cold_sets = [g] + [tuple(t.clone() for t in g) for _ in range(ncopies - 1)]
-    us_cold = time_gemm(rfk, cold_sets, args.steps, args.warmup, stream)
+    us_cold = time_gemm(rfk, cold_sets, max(args.steps, 50), max(args.warmup, 50), stream)
     del cold_sets
-    flop = 2.0 * m * n * k
-    tflops = flop / us / 1e6
-    gbs = algorithmic_bytes(m, n, k) / us / 1e3
-    cfg = rfk.select_config(m, n, k)
-    mfma_bound = flop / (PEAK_FP8_TFLOPS * 1e12) >= algorithmic_bytes(m, n, k) / (PEAK_HBM_GBS * 1e9)
-    if mfma_bound:
-        roofline = {"bound": "mfma", "achieved": round(tflops, 2), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
-                    "frac": round(tflops / PEAK_FP8_TFLOPS, 4), "traffic": None}
-    else:
-        roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                    "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}
-    # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, scaled by a copy
-    # kernel (profiles/gemm_fp8_blockscale_persistent_C2_hbm_traffic.txt); only known for the headline plan
-    if args.config == "C2" and (cfg.variant, cfg.split_k, cfg.stream_k) == (0, 1, 2):
-        roofline["traffic"] = TRAFFIC_C2_BYTES
-        roofline["traffic_note"] = TRAFFIC_C2_NOTE
-    schedule = {0: "gemm_fp8_blockscale_tile", 1: "gemm_fp8_blockscale_streamk", 2: "gemm_fp8_blockscale_persistent"}
-    roofline["kernel"] = "%s (variant %d, split_k %d)" % (schedule.get(cfg.stream_k, "?"), cfg.variant, cfg.split_k)
+    roofline = dict(rec["roofline"])
+    roofline["kernel"] = rec["kernel"]
     roofline["avg_launch_us"] = round(us, 2)
     roofline["algorithmic_flop_per_launch"] = flop
     roofline["algorithmic_bytes_per_launch"] = algorithmic_bytes(m, n, k)
@@ -224,20 +325,25 @@ def main():
     out = {
         "metric": "TFLOP/s per blockscaled fp8 GEMM (M=%d,N=%d,K=%d)" % (m, n, k),
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "settle_launches": rec["settle_launches"],
         "ms_per_step": round(us / 1e3, 5), "us_per_gemm": round(us, 2),
         "us_min": round(samples[0], 2), "us_median": round(samples[len(samples) // 2], 2),
+        "cold_clock_burst": {"us_per_gemm": round(us_burst, 2), "tflops": round(flop / us_burst / 1e6, 2),
+                             "note": "the first %d launches of the process after %d warm-up launches: shader clock and "
+                                     "board power have not reached their state under load" % (args.steps, args.warmup)},
         "cold_operands": {"us_per_gemm": round(us_cold, 2), "tflops": round(flop / us_cold / 1e6, 2),
                           "note": "%d operand sets in rotation (%.0f MB > 256 MB Infinity Cache)"
                                   % (ncopies, ncopies * set_bytes / 1e6)},
         "pct_fp8_mfma_peak": round(100 * tflops / PEAK_FP8_TFLOPS, 2),
-        "achieved_hbm_gbs_algorithmic": round(gbs, 1),
+        "achieved_hbm_gbs_algorithmic": rec["gbs_algorithmic"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3fn",
         "data": "synthetic (seeded N(0,1) fp32 -> e4m3fn, amax/448 block scales), random inputs resident in HBM",
         "config": {"workload": "%s: blockscaled fp8 GEMM M=%d N=%d K=%d, a[K][M] b[K][N] fp8, fp32 scales, bf16 C"
-                               % (args.config, m, n, k),
-                   "plan": {"variant": cfg.variant, "split_k": cfg.split_k, "group_m": cfg.group_m, "stream_k": cfg.stream_k},
+                               % (headline, m, n, k),
+                   "plan": rec["plan"],
                    "device": prop.name, "compute_units": prop.multi_processor_count, "clock_mhz": clock_mhz,
-                   "derived_fp8_peak_tflops": round(derived_peak, 1), "input_generation_s": round(gen_s, 2)},
+                   "derived_fp8_peak_tflops": round(derived_peak, 1), "input_generation_s": round(gen_s, 2),
+                   "kernel_source_sha": kernel_source_sha()},
         "roofline": roofline,
     }
 
@@ -245,46 +351,34 @@ def main():
         out["clock_under_load"] = clock_under_load(rfk, g, 0.6, us)
 
     if not args.no_cpu:
-        # CPU baseline = the oracle's torch restatement of the reference path (dequantise, fp32 matmul, bf16)
-        # on the host cores, whole workload, one timed run after a small warm-up. Also the parity gate.
-        a, b, sa, sb, c = data
-        warm = (a[:128], b, sa[:128], sb, torch.zeros((128, n), dtype=torch.bfloat16))
-        rk.ref_kernel(warm)
-        cpu_s = float("inf")
-        for _ in range(3):
-            t0 = time.perf_counter()
-            expect = rk.ref_kernel((a, b, sa, sb, torch.zeros((m, n), dtype=torch.bfloat16)))
-            cpu_s = min(cpu_s, time.perf_counter() - t0)
         out["cpu_baseline"] = {"value": round(flop / cpu_s / 1e12, 4), "unit": "TFLOP/s",
                                "cores": torch.get_num_threads(), "kind": "port", "seconds": round(cpu_s, 2),
                                "host_cpu_count": os.cpu_count(),
-                               "sample": "whole %s workload, best of 3 runs (dequantise + fp32 matmul + bf16 cast), torch CPU" % args.config}
-        out["parity"] = parity_report(rfk, cref, rk, data, g, stream, expect)
+                               "sample": "whole %s workload, best of 3 runs (dequantise + fp32 matmul + bf16 cast), torch CPU" % headline}
+        out["parity"] = rec["parity"]
+
+    if args.config is None:
+        # all five configurations: settled time, roofline fraction and the same correctness gate
+        print("%-3s %-16s %9s %9s %6s %6s %9s %9s  %s" % ("cfg", "shape", "us", "TFLOP/s", "bound", "frac", "bad@1e-2",
+              "bad@1e-3", "plan"), file=sys.stderr)
+        out["all_configs"] = {}
+        for name in sorted(CONFIGS):
+            if name == headline:
+                r = {x: rec[x] for x in rec if x != "parity"}
+                if "parity" in rec:
+                    r["parity"] = {x: rec["parity"][x] for x in ("mismatches", "mismatches_at_reference_atol_1e-3",
+                                                                  "max_abs_err", "elements", "pass")}
+            else:
+                r = measure_config(rfk, cref, rk, name, args.steps, args.warmup, stream, not args.no_cpu,
+                                   min(args.settle, 0.25))
+            out["all_configs"][name] = r
+            par = r.get("parity")
+            print("%-3s %-16s %9.2f %9.1f %6s %6.3f %9s %9s  %r" % (
+                name, "%dx%dx%d" % tuple(r["shape"]), r["us_per_gemm"], r["tflops"], r["roofline"]["bound"],
+                r["roofline"]["frac"], par["mismatches"] if par else "-",
+                par["mismatches_at_reference_atol_1e-3"] if par else "-", r["plan"]), file=sys.stderr)
 
     if args.all:
-        # the other configurations: time + the same correctness gate (stderr table, summary in the JSON line)
-        print("%-3s %-20s %10s %10s %8s %10s %8s %10s %10s  %s" % ("cfg", "shape", "us", "TFLOP/s", "%peak", "GB/s(alg)",
-              "bad@1e-2", "bad@1e-3", "err_fp64", "plan"), file=sys.stderr)
-        out["all_configs"] = {}
-        for name, (mm, nn, kk, sd) in CONFIGS.items():
-            dd = rk.generate_input_blockquant(mm, nn, kk, sd)
-            gg = to_gpu(dd)
-            u = time_gemm(rfk, [gg], args.steps, args.warmup, stream)
-            tf = 2.0 * mm * nn * kk / u / 1e6
-            gb = algorithmic_bytes(mm, nn, kk) / u / 1e3
-            rec = {"us_per_gemm": round(u, 2), "tflops": round(tf, 1), "pct_fp8_mfma_peak": round(100 * tf / PEAK_FP8_TFLOPS, 2),
-                   "gbs_algorithmic": round(gb, 1), "pct_hbm_peak": round(100 * gb / PEAK_HBM_GBS, 2)}
-            par = None
-            if not args.no_cpu:
-                par = parity_report(rfk, cref, rk, dd, gg, stream)
-                rec["parity"] = par
-            out["all_configs"][name] = rec
-            err_key = [x for x in (par or {}) if x.startswith("max_abs_err_vs_fp64")]
-            print("%-3s %-20s %10.2f %10.1f %8.2f %10.1f %8s %10s %10s  %r" % (
-                name, "%dx%dx%d" % (mm, nn, kk), u, tf, 100 * tf / PEAK_FP8_TFLOPS, gb,
-                par["mismatches"] if par else "-", par["mismatches_at_reference_atol_1e-3"] if par else "-",
-                par[err_key[0]] if par else "-", rfk.select_config(mm, nn, kk)), file=sys.stderr)
-            del gg, dd
         # the block quantisers that produce the operands (HBM-bound: source read once, fp8 + scales written once)
         out["quantisers"] = {}
         for label, fn, rows in (("quantize_a", rfk.quantize_a, m), ("quantize_b", rfk.quantize_b, n)):
