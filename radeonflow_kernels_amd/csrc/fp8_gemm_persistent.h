@@ -55,14 +55,30 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
     const int my_tiles =                                                                // >= 1: grid <= T
         __builtin_amdgcn_readfirstlane((T - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x);
 
-    // origin of this workgroup's r-th tile; past the end it repeats the last one (prefetches that nobody uses)
+    // Origin of this workgroup's r-th tile; past the end it repeats the last one (prefetches that nobody uses). The map
+    // from tile ordinal to tile costs a handful of integer divisions on the vector unit, and the two load cursors and
+    // the store each need it once per tile: with two K blocks per tile that was a tenth of the launch (6144 x 7168 x
+    // 256: 25.4 -> 23.2 us). So lane r works out the origin of tile r once, before the loop, and a tile boundary only
+    // reads that lane.
+    int m0_of_lane, n0_of_lane;
+    {
+        int tm, tn;
+        const int r = lane < my_tiles - 1 ? lane : my_tiles - 1;
+        tile_of_block(blockIdx.x + r * gridDim.x, T, tiles_m, tiles_n, group_m, true, tm, tn);
+        m0_of_lane = tm * BM;
+        n0_of_lane = tn * BN;
+    }
     auto tile_origin = [&](int r, int &m0, int &n0) {
         if (r > my_tiles - 1) r = my_tiles - 1;
-        int tm, tn;
-        tile_of_block(blockIdx.x + r * gridDim.x, T, tiles_m, tiles_n, group_m, true, tm, tn);
-        // the divisions above run on the vector unit; the origins feed scalar base pointers
-        m0 = __builtin_amdgcn_readfirstlane(tm * BM);
-        n0 = __builtin_amdgcn_readfirstlane(tn * BN);
+        if (r < 64) {
+            m0 = __builtin_amdgcn_readlane(m0_of_lane, r);
+            n0 = __builtin_amdgcn_readlane(n0_of_lane, r);
+        } else {
+            int tm, tn;
+            tile_of_block(blockIdx.x + r * gridDim.x, T, tiles_m, tiles_n, group_m, true, tm, tn);
+            m0 = __builtin_amdgcn_readfirstlane(tm * BM);
+            n0 = __builtin_amdgcn_readfirstlane(tn * BN);
+        }
     };
 
     // ---- global -> LDS: per-lane offsets inside a K block, relative to the tile origin (see tile_mainloop) ----
