@@ -452,7 +452,7 @@ def main():
         print("C2 launch time by operand bits: %r" % (out["operand_bits"],), file=sys.stderr)
         # what the chip sustains on the same MFMA instruction from registers alone (clock under its power limit);
         # run as a child process once the GEMM work above is done
-        probe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "radeonflow_kernels_amd", "lib", "mfma_ceiling")
+        probe = os.path.join(ROOT, "bench_probes", "mfma_ceiling")
         if os.path.exists(probe):
             import subprocess
             torch.cuda.synchronize()
@@ -460,6 +460,8 @@ def main():
             if r.returncode == 0:
                 out["mfma_ceiling"] = json.loads(r.stdout.strip().splitlines()[-1])
                 out["mfma_ceiling"]["gemm_pct_of_normal_ceiling"] = round(100 * out["value"] / out["mfma_ceiling"]["normal"], 2)
+                out["mfma_ceiling"]["gemm_pct_of_ceiling_with_folds_and_lds_reads"] = round(
+                    100 * out["value"] / out["mfma_ceiling"]["normal_with_folds_and_lds_reads"], 2)
                 print("register-only MFMA ceiling: %r" % (out["mfma_ceiling"],), file=sys.stderr)
             else:
                 print("mfma_ceiling failed: %s" % r.stderr.strip(), file=sys.stderr)

@@ -2,6 +2,8 @@
 
 hipcc cross-compiles without a GPU. The library is written in-tree to radeonflow_kernels_amd/lib/.
 Run:  python -m radeonflow_kernels_amd.build
+(The native test harness and the benchmark's probe have build scripts of their own: tests/checker/build.py,
+bench_probes/build.py; __graft_entry__.build() runs all three.)
 """
 import os
 import shutil
@@ -44,39 +46,8 @@ def build_lib(verbose=False):
     return LIB_PATH
 
 
-def build_checker(verbose=False):
-    """tests/checker/gemm_checker: native harness (test infrastructure; links the C oracle, dlopens libgemm.so)."""
-    root = os.path.dirname(HERE)
-    src = os.path.join(root, "tests", "checker", "gemm_checker.cpp")
-    oracle = os.path.join(root, "oracle", "fp8_blockscale_oracle.c")
-    out = os.path.join(root, "tests", "checker", "gemm_checker")
-    obj = os.path.join(root, "tests", "checker", "oracle.o")
-    _run(["gcc", "-O2", "-fopenmp", "-std=c11", "-ffp-contract=off", "-c", oracle, "-o", obj])
-    rocm = os.path.dirname(os.path.dirname(os.path.realpath(hipcc())))
-    # host-only program: plain g++ against the HIP runtime library
-    cmd = ["g++", "-O2", "-std=c++17", "-fopenmp", "-D__HIP_PLATFORM_AMD__", "-I" + os.path.join(rocm, "include"),
-           "-o", out, src, obj, "-L" + os.path.join(rocm, "lib"), "-lamdhip64", "-ldl", "-lm",
-           "-Wl,-rpath," + os.path.join(rocm, "lib"), "-Wl,-rpath,$ORIGIN/../../radeonflow_kernels_amd/lib"]
-    res = _run(cmd)
-    if verbose and res:
-        print(res)
-    return out
-
-
-def build_probe(verbose=False):
-    """lib/mfma_ceiling: register-only MFMA throughput of the whole chip (bench.py --all reports it beside the GEMM)."""
-    os.makedirs(LIB_DIR, exist_ok=True)
-    out = os.path.join(LIB_DIR, "mfma_ceiling")
-    res = _run([hipcc()] + HIPCC_FLAGS + ["-o", out, os.path.join(CSRC, "mfma_ceiling.hip")])
-    if verbose and res:
-        print(res)
-    return out
-
-
 def build_all(verbose=False):
     build_lib(verbose)
-    build_probe(verbose)
-    build_checker(verbose)
 
 
 if __name__ == "__main__":

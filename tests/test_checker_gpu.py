@@ -10,7 +10,7 @@ CHECKER = os.path.join(HERE, "checker", "gemm_checker")
 
 @pytest.mark.gpu
 def test_native_checker_single_run_mode_passes_all_cases():
-    assert os.path.exists(CHECKER), "build it with python -m radeonflow_kernels_amd.build"
+    assert os.path.exists(CHECKER), "build it with python tests/checker/build.py"
     p = subprocess.run([CHECKER, "-b"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=900)
     print(p.stdout)
     assert p.returncode == 0, p.stdout
