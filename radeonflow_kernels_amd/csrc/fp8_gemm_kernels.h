@@ -490,7 +490,9 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 // non-temporal hints measured slower than either).
 __device__ __forceinline__ void store_c16(uint16_t *p, const uint4 &v) {
     const u32x4 w = {v.x, v.y, v.z, v.w};
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" :: "v"(p), "v"(w) : "memory");
+    // A store of more than 8 bytes reads its data registers a little after it has been issued; the compiler keeps
+    // vector instructions that overwrite them away from its own stores, but it does not look inside this statement.
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" :: "v"(p), "v"(w) : "memory");
 }
 
 // Stores a wave's accumulators as bf16 into C, masked at the M and N edges. In the MFMA layout a lane owns 4
@@ -563,6 +565,54 @@ __device__ __forceinline__ void store_tile_bf16(const f32x4 (&acc)[BM / WAVES_M 
                 const int m = m0 + wm * G::WM + h * ROWS + r;
                 const int n = n0 + wn * G::WN + cb / 2;
                 if (m < M && n < N) store_c16(C + (size_t)m * N + n, v);
+            }
+        }
+    }
+}
+
+// The same for whole tiles (no edge masks) with the passes overlapped: one m-tile per pass through a private region
+// of the wave, and the global stores of a pass are issued only after the next pass's LDS traffic. LDS executes a
+// wave's instructions in order, so a pass may overwrite the region as soon as the previous pass's reads have been
+// issued; only the stores wait for read data, and by then a later pass's conversions and LDS instructions have
+// covered that latency. (With read -> store -> next write in program order a 256 x 256 tile's epilogue took 1.6 us
+// on an otherwise idle chip, nearly all of it eight LDS round trips.)
+// The staging region is written 8 bytes and read 16 bytes at a time: both through types that may alias anything, so
+// that the compiler keeps the writes (to its type rules an 8-byte vector store is never read by a 16-byte vector
+// load) and keeps them in order with the reads.
+typedef uint32_t staged_u32x2 __attribute__((ext_vector_type(2), may_alias));
+typedef uint32_t staged_u32x4 __attribute__((ext_vector_type(4), may_alias));
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+__device__ __forceinline__ void store_whole_tile_bf16(const f32x4 (&acc)[BM / WAVES_M / 16][BN / WAVES_N / 16],
+                                                      uint16_t *__restrict__ C, int N, int m0, int n0, uint8_t *staging) {
+    using G = TileGeom<BM, BN, WAVES_M, WAVES_N>;
+    constexpr int ROW = G::WN * 2 + 16;                  // bytes per staged row
+    constexpr int LPR = G::WN * 2 / 16;                  // lanes per row on the way out (16 bytes each)
+    static_assert(64 % LPR == 0 && 16 % (64 / LPR) == 0, "a store instruction covers whole rows of one m-tile");
+    constexpr int RPI = 64 / LPR, NI = 16 / RPI;         // rows per store instruction, instructions per m-tile
+    int vz;                                              // see store_tile_bf16
+    asm volatile("v_mov_b32 %0, 0" : "=v"(vz));
+    const int lane = (threadIdx.x & 63) + vz, wave = threadIdx.x >> 6, L = lane & 15, g = lane >> 4;
+    const int wm = wave % WAVES_M, wn = wave / WAVES_M;
+    uint8_t *region = staging + wave * (16 * ROW);
+    uint16_t *out = C + (size_t)(m0 + wm * G::WM + lane / LPR) * N + n0 + wn * G::WN + (lane % LPR) * 8;
+    staged_u32x4 v[2][NI];
+#pragma unroll
+    for (int j = 0; j <= G::TM; j++) {
+        if (j < G::TM) {
+#pragma unroll
+            for (int i = 0; i < G::TN; i++) {            // lane holds C[16j + L][16i + 4g .. +3]
+                const staged_u32x2 w = {pack_bf16x2(acc[j][i][0], acc[j][i][1]), pack_bf16x2(acc[j][i][2], acc[j][i][3])};
+                *(staged_u32x2 *)(region + L * ROW + (16 * i + 4 * g) * 2) = w;
+            }
+#pragma unroll
+            for (int q = 0; q < NI; q++)
+                v[j & 1][q] = *(const staged_u32x4 *)(region + (q * RPI + lane / LPR) * ROW + (lane % LPR) * 16);
+        }
+        if (j > 0) {
+#pragma unroll
+            for (int q = 0; q < NI; q++) {
+                const staged_u32x4 x = v[(j - 1) & 1][q];
+                store_c16(out + (size_t)((j - 1) * 16 + q * RPI) * N, make_uint4(x[0], x[1], x[2], x[3]));
             }
         }
     }

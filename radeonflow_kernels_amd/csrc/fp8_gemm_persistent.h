@@ -313,8 +313,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
 #pragma unroll
             for (int e = 0; e < 4; e++) acc[ju][iu][e] = __builtin_fmaf(s[TM - 1], pring[u % PR][e], acc[ju][iu][e]);
         }
-        store_tile_bf16<BM, BN, WAVES_M, WAVES_N, P::STORE_PASSES, false>(acc, C, M, N, m0_cur, n0_cur,
-                                                                          lds + P::STAGING_OFF);
+        store_whole_tile_bf16<BM, BN, WAVES_M, WAVES_N>(acc, C, N, m0_cur, n0_cur, lds + P::STAGING_OFF);
 #pragma unroll
         for (int j = 0; j < TM; j++)
 #pragma unroll
