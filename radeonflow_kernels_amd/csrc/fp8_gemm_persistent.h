@@ -250,11 +250,17 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
         advance(2, c2_r, c2_kb);
         c1_r = 0; c1_kb = 1;
         seek(1, 0, 1);
+        // like every first K block of a tile, the one that follows finds cursor 1's loads already issued
+#pragma unroll
+        for (int d = TN; d < NDMA; d++) issue_dma(d, 1, dsrc[d]);
     }
 
     // one K block of the current tile; cur = the LDS stage it reads
-    auto k_block = [&](auto cur_c) {
+    // first_c: the first K block of a tile, whose cursor-1 loads have been issued already (before the previous tile's
+    // store, see below)
+    auto k_block = [&](auto cur_c, auto first_c) {
         constexpr int cur = decltype(cur_c)::value, nxt = 1 - cur;
+        constexpr bool first = decltype(first_c)::value != 0;
         const float s_last = s[TM - 1];
 #pragma unroll
         for (int j = 0; j < TM; j++) s[j] = sraw[j] * sb_raw;
@@ -271,7 +277,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
                 bfrag[i], afrag[j & 1], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
             asm volatile("" : "+v"(pring[t % PR]));
             __builtin_amdgcn_sched_barrier(0);
-            if (t + TN < NDMA) issue_dma(t + TN, nxt, dsrc[t + TN]);                       // cursor 1
+            if (!first && t + TN < NDMA) issue_dma(t + TN, nxt, dsrc[t + TN]);             // cursor 1
             if (t >= BAR_SLOT && t - BAR_SLOT < NDMA && t - BAR_SLOT < TN)
                 issue_dma(t - BAR_SLOT, cur, dsrc[t - BAR_SLOT]);                          // cursor 2
             if (j + 1 < TM) {
@@ -301,9 +307,11 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
     };
 
     for (int r = 0; r < my_tiles; r++) {
-        for (int kb = 0; kb < QK; kb += 2) {
-            k_block(IntTag<0>{});
-            k_block(IntTag<1>{});
+        k_block(IntTag<0>{}, IntTag<1>{});
+        k_block(IntTag<1>{}, IntTag<0>{});
+        for (int kb = 2; kb < QK; kb += 2) {
+            k_block(IntTag<0>{}, IntTag<0>{});
+            k_block(IntTag<1>{}, IntTag<0>{});
         }
         // the tile is complete: fold what the last K block still owes, store, start the next tile from zero. The
         // operands of the next tile's first K block are already in registers, its second block is on its way.
@@ -313,6 +321,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
 #pragma unroll
             for (int e = 0; e < 4; e++) acc[ju][iu][e] = __builtin_fmaf(s[TM - 1], pring[u % PR][e], acc[ju][iu][e]);
         }
+        // The rest of the next tile's second K block (cursor 1; stage 1 is free since the last barrier) is asked for
+        // before this tile's stores and not in the first slots of the next K block: the memory pipeline of the CU
+        // takes instructions in order, and loads queued behind 128 KB of stores held up every wave at the start of
+        // the next tile (with two K blocks per tile: 0.7 us of each tile's 4.4).
+#pragma unroll
+        for (int d = TN; d < NDMA; d++) issue_dma(d, 1, dsrc[d]);
         store_whole_tile_bf16<BM, BN, WAVES_M, WAVES_N>(acc, C, N, m0_cur, n0_cur, lds + P::STAGING_OFF);
 #pragma unroll
         for (int j = 0; j < TM; j++)
