@@ -282,6 +282,7 @@ def main():
     ap.add_argument("--all", action="store_true", help="also quantisers, grouped form, operand bits, MFMA ceiling")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity gate")
     ap.add_argument("--settle", type=float, default=SETTLE_SECONDS, help="seconds of launches before the timed region")
+    ap.add_argument("--no-clock", action="store_true", help="skip the 0.6 s clock and power read-out (shorter profiler traces)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (output tiles are independent: "
@@ -347,8 +348,9 @@ def main():
         "roofline": roofline,
     }
 
-    with torch.cuda.stream(stream):
-        out["clock_under_load"] = clock_under_load(rfk, g, 0.6, us)
+    if not args.no_clock:
+        with torch.cuda.stream(stream):
+            out["clock_under_load"] = clock_under_load(rfk, g, 0.6, us)
 
     if not args.no_cpu:
         out["cpu_baseline"] = {"value": round(flop / cpu_s / 1e12, 4), "unit": "TFLOP/s",
@@ -432,6 +434,35 @@ def main():
                         "us": round(u, 2), "tflops": round(tf, 1), "pct_fp8_mfma_peak": round(100 * tf / PEAK_FP8_TFLOPS, 2)}
             print("%s %s: %.2f us  %.1f TFLOP/s (%.1f %% of peak)" % (key, out[key]["workload"], u, tf,
                   100 * tf / PEAK_FP8_TFLOPS), file=sys.stderr)
+        # arbitrary sizes again, with the activations quantised straight into the padded layout (quantize_a_grouped):
+        # no staging copy at all
+        offs_any = [0] + [int(x) for x in cuts_any] + [8192]
+        xg = torch.randn((gm, gk), device="cuda", dtype=torch.bfloat16)
+        with torch.cuda.stream(stream):
+            a_pad, sa_pad = rfk.quantize_a_grouped(xg, offs_any)
+            for _ in range(args.warmup // 4 + 5):
+                rfk.fp8_mm_grouped_padded(a_pad, gb, sa_pad, gsb, gc, offs_any)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(50):
+                rfk.fp8_mm_grouped_padded(a_pad, gb, sa_pad, gsb, gc, offs_any)
+            e1.record(stream)
+            stream.synchronize()
+            u = e0.elapsed_time(e1) * 1e3 / 50
+            e0.record(stream)
+            for _ in range(20):
+                rfk.quantize_a_grouped(xg, offs_any)
+            e1.record(stream)
+            stream.synchronize()
+            uq = e0.elapsed_time(e1) * 1e3 / 20
+        tf = 2.0 * gm * gn * gk / u / 1e6
+        out["grouped_any_sizes_padded_layout"] = {
+            "workload": out["grouped_any_sizes"]["workload"] + ", activations written by quantize_a_grouped",
+            "us": round(u, 2), "tflops": round(tf, 1), "pct_fp8_mfma_peak": round(100 * tf / PEAK_FP8_TFLOPS, 2),
+            "quantize_a_grouped_bf16_us": round(uq, 2)}
+        print("grouped_any_sizes_padded_layout: %.2f us  %.1f TFLOP/s (quantize_a_grouped bf16 -> padded layout: %.2f us, "
+              "includes the allocation of its outputs by torch)" % (u, tf, uq), file=sys.stderr)
+        del xg, a_pad, sa_pad
         # the same launch with other operand bits (same shapes, scales and plan): the chip's clock under load depends
         # on how many bits toggle, so the time does too
         out["operand_bits"] = {"quantised_normal_us": round(us, 2)}

@@ -153,6 +153,24 @@ void rf_gemm_destroy(void);
 int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const float *bs, void *c, const int *row_offsets,
                         int groups, int n, int k, int variant, hipStream_t stream);
 
+/* The grouped form without the staging copy: a and as already hold every group from a multiple of 16 rows on.
+ *   padded_offsets[g] = sum over earlier groups of their row counts rounded up to 16 (rf_grouped_padded_offsets writes
+ *   groups + 1 of them on the host; M_pad = padded_offsets[groups]);
+ *   a  fp8 [K][M_pad], as fp32 [K/128][M_pad]: group g's rows from column padded_offsets[g] on, anything in the padding
+ *   (rf_quantize_a_grouped_* writes zeros with scale 1); b, bs, c and row_offsets as for rf_fp8_gemm_grouped (c holds
+ *   the true rows back to back). Needs N % 16 == 0 and 16-byte aligned a, b, c (RF_ERR_BAD_CONFIG otherwise).
+ * rf_quantize_a_grouped_*: x is [M_total][K] row-major (the groups' rows back to back, row_offsets on the host);
+ * writes a and as in that padded layout in one pass, so that token counts per expert that are not multiples of 16
+ * cost no extra pass over A (the staging copy of rf_fp8_gemm_grouped is 25-40 us for 57 MB of A). The reference has
+ * no counterpart: its expert GEMMs are fp16 (src/moe/moe.cpp:213-248). */
+int rf_grouped_padded_offsets(const int *row_offsets, int groups, int *padded_offsets);
+int rf_quantize_a_grouped_f32(const float *x, const int *row_offsets, int groups, int k, void *a, float *as,
+                              hipStream_t stream);
+int rf_quantize_a_grouped_bf16(const void *x, const int *row_offsets, int groups, int k, void *a, float *as,
+                               hipStream_t stream);
+int rf_fp8_gemm_grouped_padded(const void *a, const void *b, const float *as, const float *bs, void *c,
+                               const int *row_offsets, int groups, int n, int k, int variant, hipStream_t stream);
+
 /* Block quantisers: the step before the GEMM, on the GPU. No counterpart in the reference, whose harness draws
  * fp8 bytes and scales directly (tests/gemm/gemm_test.cpp:64-99); they implement the recipe its callers use:
  * scale = amax/448 over a block (1 if the block is all zero), value = e4m3fn_rne(x / scale).

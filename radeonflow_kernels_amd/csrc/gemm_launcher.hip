@@ -932,8 +932,13 @@ long grouped_tiles(const GroupedVariant &v, const int *row_offsets, int groups, 
 
 extern "C" {
 
-int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const float *bs, void *c, const int *row_offsets,
-                        int groups, int n, int k, int variant, hipStream_t stream) {
+}  // extern "C"
+
+namespace {
+// prepadded: a and as already hold every group from a multiple of 16 rows on (the layout rf_quantize_a_grouped_* writes
+// and rf_grouped_padded_offsets describes); otherwise they hold the groups back to back as row_offsets says.
+int grouped_gemm(const void *a, const void *b, const float *as, const float *bs, void *c, const int *row_offsets,
+                 int groups, int n, int k, int variant, hipStream_t stream, bool prepadded) {
     g_last_error.clear();
     if (!row_offsets) return fail(RF_ERR_NULL_POINTER, "row_offsets is null");
     if (groups < 1 || groups > rf::kMaxGroups)
@@ -959,6 +964,11 @@ int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const flo
     const bool direct = n % 16 == 0 && ((uintptr_t)b % 16) == 0 && ((uintptr_t)c % 16) == 0;
     bool stage = ((uintptr_t)a % 16) != 0;
     for (int g = 0; g <= groups; g++) stage = stage || row_offsets[g] % 16 != 0;
+    if (prepadded) {
+        if (!direct || ((uintptr_t)a % 16) != 0)
+            return fail(RF_ERR_BAD_CONFIG, "the padded layout needs N % 16 == 0 and 16-byte aligned a, b and c");
+        stage = false;
+    }
     if (!direct || (stage && (double)m_total * n * k < kPadThresholdMacs)) {
         // ragged N, unaligned weights or output, or next to no work: the bounds-checked kernel, one launch per
         // non-empty group
@@ -1001,6 +1011,15 @@ int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const flo
         RF_HIP(hipGetLastError());
         a = pad;
         as = (const float *)(pad + a_bytes);
+    } else if (prepadded) {
+        int at = 0;
+        for (int g = 0; g < groups; g++) {
+            table.row_start[g] = at;
+            at += (row_offsets[g + 1] - row_offsets[g] + 15) / 16 * 16;
+        }
+        for (int g = groups; g <= rf::kMaxGroups; g++) table.row_start[g] = at;
+        for (int g = 0; g <= rf::kMaxGroups; g++) table.out_row_start[g] = row_offsets[g < groups ? g : groups];
+        m_rows = at;
     } else {
         for (int g = 0; g <= rf::kMaxGroups; g++)
             table.row_start[g] = table.out_row_start[g] = row_offsets[g < groups ? g : groups];
@@ -1043,6 +1062,74 @@ int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const flo
                        bs, (uint16_t *)c, m_rows, n, k, groups, tiles_n, 8, table);
     RF_HIP(hipGetLastError());
     return RF_OK;
+}
+
+template <bool IN_BF16>
+int quantize_a_grouped(const void *x, const int *row_offsets, int groups, int k, void *a, float *as, hipStream_t stream) {
+    g_last_error.clear();
+    if (!row_offsets) return fail(RF_ERR_NULL_POINTER, "row_offsets is null");
+    if (groups < 1 || groups > rf::kQuantMaxGroups || k < rf::BK || k % rf::BK != 0 || row_offsets[0] != 0)
+        return fail(RF_ERR_BAD_SHAPE, "unsupported shape (need 1 <= groups <= 256, K a positive multiple of 128, row_offsets[0] == 0)");
+    rf::QuantGroups tab;
+    int at = 0;
+    for (int g = 0; g < groups; g++) {
+        if (row_offsets[g + 1] < row_offsets[g]) return fail(RF_ERR_BAD_SHAPE, "row_offsets must not decrease");
+        tab.pad_start[g] = at;
+        tab.src_start[g] = row_offsets[g];
+        at += (row_offsets[g + 1] - row_offsets[g] + 15) / 16 * 16;
+    }
+    for (int g = groups; g <= rf::kQuantMaxGroups; g++) { tab.pad_start[g] = at; tab.src_start[g] = row_offsets[groups]; }
+    tab.groups = groups;
+    if (at == 0) return RF_OK;
+    if (!x || !a || !as) return fail(RF_ERR_NULL_POINTER, "null device pointer");
+    if ((uintptr_t)x % 16 != 0 || (uintptr_t)a % 16 != 0 || (uintptr_t)as % 4 != 0)
+        return fail(RF_ERR_BAD_CONFIG, "source and a must be 16-byte aligned, scales 4-byte aligned");
+    State &s = state();
+    {
+        std::lock_guard<std::mutex> lock(shared().mu);
+        int rc = ensure_device_info(s);
+        if (rc != RF_OK) return rc;
+    }
+    hipLaunchKernelGGL((rf::quantize_block128_grouped<IN_BF16>), dim3(k / rf::BK, ceil_div(at, 128)), dim3(256), 0, stream, x,
+                       at, k, (uint8_t *)a, as, tab);
+    RF_HIP(hipGetLastError());
+    return RF_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const float *bs, void *c, const int *row_offsets,
+                        int groups, int n, int k, int variant, hipStream_t stream) {
+    return grouped_gemm(a, b, as, bs, c, row_offsets, groups, n, k, variant, stream, false);
+}
+
+int rf_fp8_gemm_grouped_padded(const void *a, const void *b, const float *as, const float *bs, void *c,
+                               const int *row_offsets, int groups, int n, int k, int variant, hipStream_t stream) {
+    return grouped_gemm(a, b, as, bs, c, row_offsets, groups, n, k, variant, stream, true);
+}
+
+int rf_grouped_padded_offsets(const int *row_offsets, int groups, int *padded_offsets) {
+    g_last_error.clear();
+    if (!row_offsets || !padded_offsets) return fail(RF_ERR_NULL_POINTER, "null pointer");
+    if (groups < 1 || groups > rf::kMaxGroups || row_offsets[0] != 0) return fail(RF_ERR_BAD_SHAPE, "unsupported groups");
+    int at = 0;
+    for (int g = 0; g < groups; g++) {
+        if (row_offsets[g + 1] < row_offsets[g]) return fail(RF_ERR_BAD_SHAPE, "row_offsets must not decrease");
+        padded_offsets[g] = at;
+        at += (row_offsets[g + 1] - row_offsets[g] + 15) / 16 * 16;
+    }
+    padded_offsets[groups] = at;
+    return RF_OK;
+}
+
+int rf_quantize_a_grouped_f32(const float *x, const int *row_offsets, int groups, int k, void *a, float *as,
+                              hipStream_t stream) {
+    return quantize_a_grouped<false>(x, row_offsets, groups, k, a, as, stream);
+}
+int rf_quantize_a_grouped_bf16(const void *x, const int *row_offsets, int groups, int k, void *a, float *as,
+                               hipStream_t stream) {
+    return quantize_a_grouped<true>(x, row_offsets, groups, k, a, as, stream);
 }
 
 int rf_cast_f32_to_e4m3fn(const float *x, size_t count, void *out, hipStream_t stream) {

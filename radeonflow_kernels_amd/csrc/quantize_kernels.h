@@ -115,10 +115,21 @@ __device__ __forceinline__ float div_by_448(float a) {
 // A thread loads 16 bytes at a time: KPT = 4 (fp32) or 8 (bf16) consecutive k of one row, so a row is spread over
 // LPR = 32 (16) neighbouring lanes; it holds RPT = 16 (8) rows, in runs of four consecutive rows (a run becomes one
 // 32-bit LDS store per k): run g of thread t starts at row g * (128 / NG) + 4 * (t / LPR).
-template <bool PER_ROW, bool IN_BF16>
-__global__ __launch_bounds__(256) void quantize_block128(const void *__restrict__ X, int R, int K,
-                                                         uint8_t *__restrict__ out, float *__restrict__ scales,
-                                                         int scale_ld, bool vector_store) {
+//
+// GROUPED (activations of several groups, for the grouped GEMM): the R rows written are the rows of a padded layout in
+// which group g starts at row pad_start[g], a multiple of 16, and holds src_start[g+1] - src_start[g] rows of X (from
+// row src_start[g]) followed by rows of zeros with scale 1 up to the next group's start. Group starts are multiples
+// of 16 and a thread's rows come in runs of four from a multiple of four, so a run lies in one group.
+constexpr int kQuantMaxGroups = 256;
+struct QuantGroups {
+    int pad_start[kQuantMaxGroups + 1];     // first row of each group in the padded layout; [groups] = R
+    int src_start[kQuantMaxGroups + 1];     // first row of each group in X; [groups] = rows of X
+    int groups;
+};
+template <bool PER_ROW, bool IN_BF16, bool GROUPED>
+__device__ __forceinline__ void quantize_block128_body(const void *__restrict__ X, int R, int K,
+                                                       uint8_t *__restrict__ out, float *__restrict__ scales,
+                                                       int scale_ld, bool vector_store, const QuantGroups &tab) {
     constexpr int KPT = IN_BF16 ? 8 : 4, LPR = 128 / KPT, RPT = 64 / KPT, NG = RPT / 4;
     constexpr int PITCH = 128 + 4;                            // LDS row (one k, 128 rows of X), padded against conflicts
     __shared__ __attribute__((aligned(16))) uint8_t tile[128 * PITCH];
@@ -129,12 +140,41 @@ __global__ __launch_bounds__(256) void quantize_block128(const void *__restrict_
     const int rb = blockIdx.y, r0 = rb * 128, kb = blockIdx.x, k0 = kb * 128;
     // All loads are issued before the first one is used: rows past R read row R-1 again (their results are never
     // stored, and they are kept out of a block-wide maximum below) instead of sitting behind a branch each.
+    // GROUPED: source row of each run of four rows and the first padded row past its group's true rows. The groups
+    // that reach into this block are found with table reads that are the same for all lanes (the block starts in
+    // group g0; at most 8 more groups of at least 16 padded rows follow inside it).
+    int run_shift[NG], run_limit[NG];
+    if constexpr (GROUPED) {
+        int lo = 0, hi = tab.groups;                          // last g with pad_start[g] <= r0 (uniform)
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (tab.pad_start[mid] <= r0) lo = mid; else hi = mid;
+        }
+#pragma unroll
+        for (int u = 0; u < NG; u++) { run_shift[u] = 0; run_limit[u] = 0; }
+        for (int g = lo; g < tab.groups && tab.pad_start[g] < r0 + 128; g++) {
+            const int ps = tab.pad_start[g], ss = tab.src_start[g], rows = tab.src_start[g + 1] - ss;
+#pragma unroll
+            for (int u = 0; u < NG; u++)
+                if (r0 + row_of(4 * u) >= ps) { run_shift[u] = ss - ps; run_limit[u] = ps + rows; }
+        }
+    }
+    const int src_rows = GROUPED ? tab.src_start[tab.groups] : R;
     uint4 raw[RPT];
 #pragma unroll
     for (int i = 0; i < RPT; i++) {
-        const int r = r0 + row_of(i), rc = r < R ? r : R - 1;
+        const int r = r0 + row_of(i);
+        int rc = r < R ? r : R - 1;
+        if constexpr (GROUPED) {
+            rc = r + run_shift[i >> 2];
+            rc = rc < src_rows ? rc : src_rows - 1;
+            rc = rc > 0 ? rc : 0;
+        }
         const size_t off = (size_t)rc * K + k0 + KPT * lane_k;
         raw[i] = IN_BF16 ? *(const uint4 *)((const uint16_t *)X + off) : *(const uint4 *)((const float *)X + off);
+        if constexpr (GROUPED) {
+            if (r >= run_limit[i >> 2]) raw[i] = make_uint4(0u, 0u, 0u, 0u);      // padding row: zeros, scale 1
+        }
     }
     float v[RPT][KPT];
 #pragma unroll
@@ -298,6 +338,20 @@ __global__ __launch_bounds__(256) void quantize_block128(const void *__restrict_
             if (r0 + c < R) out[(size_t)(k0 + k) * R + r0 + c] = tile[k * PITCH + c];
         }
     }
+}
+
+template <bool PER_ROW, bool IN_BF16>
+__global__ __launch_bounds__(256) void quantize_block128(const void *__restrict__ X, int R, int K,
+                                                         uint8_t *__restrict__ out, float *__restrict__ scales,
+                                                         int scale_ld, bool vector_store) {
+    QuantGroups none;                                         // not read
+    quantize_block128_body<PER_ROW, IN_BF16, false>(X, R, K, out, scales, scale_ld, vector_store, none);
+}
+template <bool IN_BF16>
+__global__ __launch_bounds__(256) void quantize_block128_grouped(const void *__restrict__ X, int R, int K,
+                                                                 uint8_t *__restrict__ out, float *__restrict__ scales,
+                                                                 const QuantGroups tab) {
+    quantize_block128_body<true, IN_BF16, true>(X, R, K, out, scales, R, true, tab);
 }
 
 }  // namespace rf

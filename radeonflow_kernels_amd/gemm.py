@@ -41,7 +41,8 @@ EXPORTS = ("run", "rf_fp8_gemm", "rf_fp8_gemm_ex", "rf_gemm_select_config", "rf_
            "rf_gemm_variant_info", "rf_gemm_variant_has_stream_k", "rf_gemm_variant_has_persistent", "rf_gemm_workspace_bytes", "rf_gemm_init", "rf_gemm_destroy",
            "rf_gemm_last_error", "rf_fp8_gemm_grouped", "rf_quantize_a_f32", "rf_quantize_a_bf16", "rf_quantize_b_f32", "rf_quantize_b_bf16",
            "rf_cast_f32_to_e4m3fn", "rf_gemm_load_plans", "rf_gemm_clear_plans", "rf_fp8_gemm_time", "rf_fp8_gemm_static",
-           "rf_gemm_static_scratch_bytes")
+           "rf_gemm_static_scratch_bytes", "rf_grouped_padded_offsets", "rf_quantize_a_grouped_f32",
+           "rf_quantize_a_grouped_bf16", "rf_fp8_gemm_grouped_padded")
 
 
 def lib():
@@ -86,6 +87,14 @@ def lib():
         L.rf_gemm_last_error.restype = ctypes.c_char_p
         L.rf_fp8_gemm_grouped.argtypes = [ctypes.c_void_p] * 5 + [ctypes.POINTER(i32), i32, i32, i32, i32, ctypes.c_void_p]
         L.rf_fp8_gemm_grouped.restype = i32
+        L.rf_fp8_gemm_grouped_padded.argtypes = [ctypes.c_void_p] * 5 + [ctypes.POINTER(i32), i32, i32, i32, i32, ctypes.c_void_p]
+        L.rf_fp8_gemm_grouped_padded.restype = i32
+        L.rf_grouped_padded_offsets.argtypes = [ctypes.POINTER(i32), i32, ctypes.POINTER(i32)]
+        L.rf_grouped_padded_offsets.restype = i32
+        for name in ("rf_quantize_a_grouped_f32", "rf_quantize_a_grouped_bf16"):
+            f = getattr(L, name)
+            f.argtypes = [ctypes.c_void_p, ctypes.POINTER(i32), i32, i32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+            f.restype = i32
         for name in ("rf_quantize_a_f32", "rf_quantize_a_bf16", "rf_quantize_b_f32", "rf_quantize_b_bf16"):
             f = getattr(L, name)
             f.argtypes = [ctypes.c_void_p, i32, i32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
@@ -175,8 +184,8 @@ def fp8_mm_grouped(a, b, a_scale, b_scale, c, row_offsets, variant=-1):
           and tuple(b.shape) == (groups, n, k) and tuple(c.shape) == (m_total, n) and c.is_contiguous()
           and (m_total <= 1 or k == 1 or a.stride() == (1, m_total)) and tuple(a_scale.shape) == (m_total, qk)
           and (m_total <= 1 or qk == 1 or a_scale.stride() == (1, m_total))
-          and b.stride() == (k * n, 1, n) and tuple(b_scale.shape) == (groups, qn, qk)
-          and (b_scale.stride() == (qk * qn, 1, qn) or qn == 1 or qk == 1) and len(row_offsets) == groups + 1)
+          and (b.stride() == (k * n, 1, n) or (groups == 1 and b.stride()[1:] == (1, n))) and tuple(b_scale.shape) == (groups, qn, qk)
+          and (b_scale.stride() == (qk * qn, 1, qn) or qn == 1 or qk == 1 or (groups == 1 and b_scale.stride()[1:] == (1, qn))) and len(row_offsets) == groups + 1)
     if not ok:
         raise ValueError("fp8_mm_grouped: operands do not have the documented dtypes / shapes / strides")
     offs = (ctypes.c_int32 * (groups + 1))(*[int(x) for x in row_offsets])
@@ -186,6 +195,65 @@ def fp8_mm_grouped(a, b, a_scale, b_scale, c, row_offsets, variant=-1):
                                        offs, groups, n, k, variant, stream)
     if rc != RF_OK:
         raise RuntimeError("rf_fp8_gemm_grouped failed (%d): %s" % (rc, last_error()))
+
+
+def grouped_padded_offsets(row_offsets):
+    """Row offsets of the padded layout: every group starts at a multiple of 16 (list of len(row_offsets) ints)."""
+    groups = len(row_offsets) - 1
+    offs = (ctypes.c_int32 * (groups + 1))(*[int(x) for x in row_offsets])
+    out = (ctypes.c_int32 * (groups + 1))()
+    rc = lib().rf_grouped_padded_offsets(offs, groups, out)
+    if rc != RF_OK:
+        raise RuntimeError("rf_grouped_padded_offsets failed (%d): %s" % (rc, last_error()))
+    return list(out)
+
+
+def quantize_a_grouped(x, row_offsets):
+    """Activations [M_total, K] (fp32 or bf16, contiguous, on the GPU) of groups that own rows row_offsets[g] ..
+    row_offsets[g+1]-1 -> (a, a_scale) in the padded layout fp8_mm_grouped_padded takes: a [M_pad, K] stride (1, M_pad),
+    a_scale [M_pad, K/128] stride (1, M_pad); padding rows hold zeros with scale 1."""
+    if x.dim() != 2 or not x.is_contiguous() or x.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("source must be a contiguous 2-D fp32 or bf16 tensor [rows, K]")
+    rows, k = x.shape
+    if k < 128 or k % 128 or int(row_offsets[-1]) != rows:
+        raise ValueError("K must be a positive multiple of 128 and row_offsets must end at the number of rows")
+    groups = len(row_offsets) - 1
+    m_pad = grouped_padded_offsets(row_offsets)[-1]
+    a = torch.empty((k, m_pad), dtype=torch.float8_e4m3fn, device=x.device)
+    a_scale = torch.empty((k // 128, m_pad), dtype=torch.float32, device=x.device)
+    offs = (ctypes.c_int32 * (groups + 1))(*[int(v) for v in row_offsets])
+    name = "rf_quantize_a_grouped_%s" % ("f32" if x.dtype == torch.float32 else "bf16")
+    stream = ctypes.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)
+    with torch.cuda.device(x.device):
+        rc = getattr(lib(), name)(x.data_ptr(), offs, groups, k, a.data_ptr(), a_scale.data_ptr(), stream)
+    if rc != RF_OK:
+        raise RuntimeError("%s failed (%d): %s" % (name, rc, last_error()))
+    return a.T, a_scale.T
+
+
+def fp8_mm_grouped_padded(a, b, a_scale, b_scale, c, row_offsets, variant=-1):
+    """fp8_mm_grouped on activations already in the padded layout (quantize_a_grouped): a [M_pad, K] stride (1, M_pad),
+    a_scale [M_pad, K/128] stride (1, M_pad); b, b_scale, c and row_offsets as for fp8_mm_grouped."""
+    m_pad, k = a.shape
+    groups, n, _ = b.shape
+    qk, qn = k // 128, (n + 127) // 128
+    m_total = int(row_offsets[-1])
+    ok = (a.dtype == torch.float8_e4m3fn and b.dtype == torch.float8_e4m3fn and c.dtype == torch.bfloat16
+          and a_scale.dtype == torch.float32 and b_scale.dtype == torch.float32 and len(row_offsets) == groups + 1
+          and m_pad == grouped_padded_offsets(row_offsets)[-1] and a.stride() == (1, m_pad)
+          and tuple(a_scale.shape) == (m_pad, qk) and (qk == 1 or a_scale.stride() == (1, m_pad))
+          and tuple(b.shape) == (groups, n, k) and (b.stride() == (k * n, 1, n) or (groups == 1 and b.stride()[1:] == (1, n)))
+          and tuple(b_scale.shape) == (groups, qn, qk) and (b_scale.stride() == (qk * qn, 1, qn) or qn == 1 or qk == 1 or (groups == 1 and b_scale.stride()[1:] == (1, qn)))
+          and tuple(c.shape) == (m_total, n) and c.is_contiguous())
+    if not ok:
+        raise ValueError("fp8_mm_grouped_padded: operands do not have the documented dtypes / shapes / strides")
+    offs = (ctypes.c_int32 * (groups + 1))(*[int(x) for x in row_offsets])
+    stream = ctypes.c_void_p(torch.cuda.current_stream(a.device).cuda_stream)
+    with torch.cuda.device(a.device):
+        rc = lib().rf_fp8_gemm_grouped_padded(a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(),
+                                              c.data_ptr(), offs, groups, n, k, variant, stream)
+    if rc != RF_OK:
+        raise RuntimeError("rf_fp8_gemm_grouped_padded failed (%d): %s" % (rc, last_error()))
 
 
 def custom_kernel(data):

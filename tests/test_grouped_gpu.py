@@ -160,3 +160,69 @@ def test_grouped_status_codes(rfk):
     assert L.rf_fp8_gemm_grouped(None, None, None, None, None, offs, 1, 128, 128, -1, None) == 2      # null pointers
     assert L.rf_fp8_gemm_grouped(None, None, None, None, None, offs, 1, 128, 100, -1, None) == 1      # bad K
     assert L.rf_fp8_gemm_grouped(None, None, None, None, None, offs, 300, 128, 128, -1, None) == 1    # too many groups
+
+
+PADDED_CASES = [([100, 37, 0, 400, 1, 16, 255], 512, 256), ([5] * 40, 256, 384), ([1000], 256, 128),
+                ([0, 0, 17], 144, 128), ([int(x) for x in np.random.default_rng(11).integers(0, 300, 48)], 768, 512)]
+
+
+@pytest.mark.parametrize("kind", ["f32", "bf16"])
+@pytest.mark.parametrize("rows,n,k", PADDED_CASES)
+def test_grouped_quantiser_writes_the_padded_layout_of_the_oracle_quantiser(rfk, rows, n, k, kind):
+    """quantize_a_grouped: every group's rows start at a multiple of 16 and equal, bit for bit, the oracle quantiser's
+    rows of the same activations (values with ties, zeros and large magnitudes among them); the padding rows hold zero
+    codes with scale 1; nothing is written past the padded matrix."""
+    rng = np.random.default_rng(sum(rows) + k)
+    offs = [0] + [int(x) for x in np.cumsum(rows)]
+    m_total = offs[-1]
+    x = (rng.standard_normal((m_total, k)) * rng.choice([1e-3, 1.0, 300.0], (m_total, 1))).astype(np.float32)
+    x[rng.random((m_total, k)) < 0.05] = 0.0
+    xt = torch.from_numpy(x).cuda()
+    if kind == "bf16":
+        xt = xt.to(torch.bfloat16)
+        x = xt.float().cpu().numpy()
+    a_ref, as_ref = cref.quantize_a(x)                          # [K][M_total], [K/128][M_total]
+    pad = rfk.grouped_padded_offsets(offs)
+    assert pad[0] == 0 and all(p % 16 == 0 for p in pad) and pad[-1] == sum((r + 15) // 16 * 16 for r in rows)
+    a, sa = rfk.quantize_a_grouped(xt, offs)
+    torch.cuda.synchronize()
+    a_np = a.T.contiguous().view(torch.uint8).cpu().numpy()     # [K][M_pad]
+    sa_np = sa.T.contiguous().cpu().numpy()
+    assert a_np.shape == (k, pad[-1]) and sa_np.shape == (k // 128, pad[-1])
+    for g, r in enumerate(rows):
+        assert np.array_equal(a_np[:, pad[g]:pad[g] + r], a_ref[:, offs[g]:offs[g + 1]]), "codes of group %d" % g
+        assert np.array_equal(sa_np[:, pad[g]:pad[g] + r], as_ref[:, offs[g]:offs[g + 1]]), "scales of group %d" % g
+        assert not a_np[:, pad[g] + r:pad[g + 1]].any() and np.all(sa_np[:, pad[g] + r:pad[g + 1]] == 1.0)
+
+
+@pytest.mark.parametrize("rows,n,k", PADDED_CASES)
+def test_grouped_gemm_on_the_padded_layout_equals_the_staged_path(rfk, rows, n, k):
+    """Activations quantised straight into the padded layout, then fp8_mm_grouped_padded: the same bits as quantising
+    them back to back and letting fp8_mm_grouped stage them, for every tile variant; rows of C outside the groups'
+    true rows do not exist and the canary behind C stays intact."""
+    rng = np.random.default_rng(sum(rows) + n)
+    offs = [0] + [int(x) for x in np.cumsum(rows)]
+    m_total, groups = offs[-1], len(rows)
+    x = torch.from_numpy(rng.standard_normal((m_total, k)).astype(np.float32)).cuda()
+    w = torch.from_numpy(rng.standard_normal((groups * n, k)).astype(np.float32)).cuda()
+    b2, sb2 = rfk.quantize_b(w)                                 # [G*N, K] stride (1, G*N): regroup into [G][K][N]
+    fp8 = torch.float8_e4m3fn
+    b = b2.T.contiguous().view(torch.uint8).view(k, groups, n).permute(1, 0, 2).contiguous().view(fp8).permute(0, 2, 1)
+    qn = (n + 127) // 128
+    if n % 128 == 0:
+        sb = sb2.T.contiguous().view(k // 128, groups, qn).permute(1, 0, 2).contiguous().permute(0, 2, 1)
+    else:                                                       # a group's blocks do not line up: one scale everywhere
+        sb = torch.full((groups, k // 128, qn), 0.01, device="cuda").permute(0, 2, 1)
+    a_flat, sa_flat = rfk.quantize_a(x)
+    a_pad, sa_pad = rfk.quantize_a_grouped(x, offs)
+    for variant in (-1, 0, 1, 2, 3, 4):
+        buf = torch.full((m_total * n + CANARY,), -7.0, dtype=torch.bfloat16, device="cuda")
+        c1 = torch.zeros((m_total, n), dtype=torch.bfloat16, device="cuda")
+        c2 = buf[: m_total * n].view(m_total, n)
+        c2.zero_()
+        rfk.fp8_mm_grouped(a_flat, b, sa_flat, sb, c1, offs, variant=variant)
+        rfk.fp8_mm_grouped_padded(a_pad, b, sa_pad, sb, c2, offs, variant=variant)
+        torch.cuda.synchronize()
+        assert torch.equal(c1.view(torch.uint16), c2.view(torch.uint16)), "variant %d" % variant
+        assert bool(c1.float().abs().sum() > 0)
+        _check_canary(buf, m_total * n)
