@@ -1080,6 +1080,10 @@ int quantize_a_grouped(const void *x, const int *row_offsets, int groups, int k,
     }
     for (int g = groups; g <= rf::kQuantMaxGroups; g++) { tab.pad_start[g] = at; tab.src_start[g] = row_offsets[groups]; }
     tab.groups = groups;
+    for (int blk = 0, g = 0; blk < rf::kQuantBlockTable; blk++) {        // last g with pad_start[g] <= 128 * blk
+        while (g + 1 < groups && tab.pad_start[g + 1] <= 128 * blk) g++;
+        tab.block_group[blk] = (unsigned short)g;
+    }
     if (at == 0) return RF_OK;
     if (!x || !a || !as) return fail(RF_ERR_NULL_POINTER, "null device pointer");
     if ((uintptr_t)x % 16 != 0 || (uintptr_t)a % 16 != 0 || (uintptr_t)as % 4 != 0)

@@ -125,7 +125,11 @@ struct QuantGroups {
     int pad_start[kQuantMaxGroups + 1];     // first row of each group in the padded layout; [groups] = R
     int src_start[kQuantMaxGroups + 1];     // first row of each group in X; [groups] = rows of X
     int groups;
+    // the group that holds the first row of each 128-row block of the padded layout, for the first kQuantBlockTable
+    // blocks (later blocks search the table): a search is eight dependent scalar loads, about as long as a block's work
+    unsigned short block_group[512];
 };
+constexpr int kQuantBlockTable = 512;
 template <bool PER_ROW, bool IN_BF16, bool GROUPED>
 __device__ __forceinline__ void quantize_block128_body(const void *__restrict__ X, int R, int K,
                                                        uint8_t *__restrict__ out, float *__restrict__ scales,
@@ -146,9 +150,13 @@ __device__ __forceinline__ void quantize_block128_body(const void *__restrict__ 
     int run_shift[NG], run_limit[NG];
     if constexpr (GROUPED) {
         int lo = 0, hi = tab.groups;                          // last g with pad_start[g] <= r0 (uniform)
-        while (hi - lo > 1) {
-            const int mid = (lo + hi) >> 1;
-            if (tab.pad_start[mid] <= r0) lo = mid; else hi = mid;
+        if (rb < kQuantBlockTable) {
+            lo = tab.block_group[rb];
+        } else {
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) >> 1;
+                if (tab.pad_start[mid] <= r0) lo = mid; else hi = mid;
+            }
         }
 #pragma unroll
         for (int u = 0; u < NG; u++) { run_shift[u] = 0; run_limit[u] = 0; }

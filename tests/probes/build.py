@@ -1,4 +1,5 @@
-"""Builds tests/probes/mfma_precision (test infrastructure: the matrix unit's summation precision, one wave).
+"""Builds the probes under tests/probes (test infrastructure): mfma_precision (the matrix unit's summation precision, one
+wave) and lds_dma_order (completion order of LDS-DMA loads).
 
 Run:  python tests/probes/build.py
 """
@@ -13,12 +14,15 @@ if ROOT not in sys.path:
 
 def build_probes(verbose=False):
     from radeonflow_kernels_amd.build import HIPCC_FLAGS, _run, hipcc
-    out = os.path.join(HERE, "mfma_precision")
     flags = [f for f in HIPCC_FLAGS if f != "-fPIC"]
-    res = _run([hipcc()] + flags + ["-o", out, os.path.join(HERE, "mfma_precision.hip")])
-    if verbose and res:
-        print(res)
-    return out
+    outs = []
+    for name in ("mfma_precision", "lds_dma_order"):
+        out = os.path.join(HERE, name)
+        res = _run([hipcc()] + flags + ["-o", out, os.path.join(HERE, name + ".hip")])
+        if verbose and res:
+            print(res)
+        outs.append(out)
+    return outs
 
 
 if __name__ == "__main__":

@@ -1,4 +1,6 @@
-"""Why a few outputs miss the reference harness's atol of 1e-3 (tests/gemm/gemm_test.cpp:202-205 of the reference) while
+"""Hardware facts the kernels and the documentation rely on, measured on the GPU by small probes under tests/probes.
+
+Why a few outputs miss the reference harness's atol of 1e-3 (tests/gemm/gemm_test.cpp:202-205 of the reference) while
 all meet the graded atol of 1e-2: the gfx950 matrix unit does not sum the 128 products of an fp8 MFMA in full fp32.
 Both statements are checked here on the GPU: the unit's precision in isolation, and what follows for the GEMM."""
 import json
@@ -80,3 +82,20 @@ def test_outputs_outside_the_reference_atol_are_explained_by_the_matrix_unit(nam
         worst = max(worst, err / bound)
         assert err <= bound, "(%d, %d): GPU %.6g, exact %.6g, error %.3g above the bound %.3g" % (r, c, got[r, c], truth, err, bound)
     print("%s: largest error / bound = %.3f" % (name, worst))
+
+
+def test_lds_dma_loads_of_a_wave_complete_in_issue_order():
+    """global_load_lds_dwordx4 loads that miss L2 (random 1 KiB pieces of a 1 GiB buffer), followed by loads that hit
+    (16-byte and 4-byte ones), then s_waitcnt vmcnt(n) with n = the number of younger loads: the older loads' data is
+    in LDS every time. (The GEMM kernels wait with vmcnt(0) only; this keeps the fact on record for pipelines with
+    more than one K block of loads in flight.)"""
+    probe = os.path.join(HERE, "probes", "lds_dma_order")
+    assert os.path.exists(probe), "build it with python tests/probes/build.py"
+    p = subprocess.run([probe, "500"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=200)
+    assert p.returncode == 0, p.stdout + p.stderr
+    lines = [l for l in p.stdout.splitlines() if " stale " in l]
+    print(p.stdout)
+    assert len(lines) == 6
+    for l in lines:
+        f = l.split()
+        assert int(f[f.index("checked") + 1]) > 10 ** 9 and int(f[f.index("stale") + 1]) == 0, l
