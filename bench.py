@@ -62,7 +62,7 @@ def measured_traffic(config, cfg):
     sources have changed since it was taken."""
     plan = "%d,%d,%d" % (cfg.variant, cfg.split_k, cfg.stream_k)
     why = "no rocprofv3 traffic summary for %s under profiles/" % config
-    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*hbm_traffic*.txt"))):
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*.txt"))):
         for line in open(path):
             if not line.startswith("@traffic"):
                 continue
