@@ -66,6 +66,24 @@ def test_every_variant_and_split(rfk, gen, m, n, k):
             assert_few_mismatches_at_reference_atol(out, exp, "variant %r split %d" % (v, split))
 
 
+@pytest.mark.parametrize("m,n", [(1024, 1536), (640, 576), (768, 2304), (2048, 384), (1040, 208)])
+def test_split_k_grid_reaches_every_tile_and_split_once(rfk, m, n):
+    """Every variant with 2 to 16 K splits (counts that divide the 16 K blocks and counts that leave the last split
+    short), on tile grids that do and do not divide by the number of XCDs: bit-exact on data whose sums are exact in
+    any order, after a launch of another problem with the same plan (partial sums of a tile or split nobody computed
+    would be that problem's)."""
+    k = 2048
+    data = exact_problem(m, n, k, seed=m + n)
+    exp = oracle_bf16(data)
+    other = to_gpu(exact_problem(m, n, k, seed=m + n + 1))
+    for v in rfk.variants():
+        for split in (2, 3, 4, 5, 8, 16):
+            cfg = rfk.GemmConfig(v["variant"], split, 3, 0)
+            rfk.fp8_mm(*other, config=cfg)                  # fills the workspace with another problem's sums
+            out = _run(rfk, data, config=cfg, canary=1024)
+            assert np.array_equal(bf16_bits(out), exp), "variant %r split %d" % (v, split)
+
+
 @pytest.mark.parametrize("m,n,k", [(256, 384, 512), (512, 576, 1024), (272, 144, 256), (16, 16, 128), (1024, 1536, 7168),
                                    (48, 80, 7168), (33, 47, 384)])
 def test_bit_exact_on_exactly_representable_data(rfk, m, n, k):
