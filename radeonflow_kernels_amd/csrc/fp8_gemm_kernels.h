@@ -837,33 +837,56 @@ __global__ __launch_bounds__(256) void reduce_splitk_bf16(const float *__restric
 // C may pack the groups more tightly than A does: group g writes out_row_start[g+1] - out_row_start[g] rows from row
 // out_row_start[g] of C, any counts, while its A rows start at row_start[g] and are padded to a multiple of 16 (the
 // host stages A that way when the caller's group sizes are not multiples of 16).
+//
+// Which workgroup computes what. The expert weights are the bulk of the bytes (one [K][N] block per group, read by
+// the few row tiles the group has), and what an XCD's workgroups read its own L2 has to fetch: with a group's tiles
+// dealt round-robin over the 8 XCDs every L2 fetches the group's A rows and several L2s the same weight tile (32
+// uneven groups, 8192 x 4096 x 7168: 2.06 GB fetched for 1.0 GB of operands; 1.28 GB with the map below). So the work
+// items are put in one line, group by group, a group's column tiles one after the other and the row tiles of a
+// column tile side by side, and the line is cut into 8 contiguous pieces with the same number of items, one per XCD.
+// An XCD then works through a few whole groups: a weight tile is fetched by one L2 and serves all row tiles of its
+// group there, and a group's A rows are fetched once (twice for a group cut by a piece boundary). Workgroup b runs
+// on XCD b % 8 and takes item number b / 8 of that XCD's piece. Equal counts, not equal estimated cost: workgroups
+// are handed out in the order of their ids, and when the XCD whose turn it is has no free CU the others wait with
+// it, so all XCDs move through their pieces at the same pace; pieces of equal estimated cost but different lengths
+// (a 128-row tile counted as 0.6 of a 256-row one) measured 12 % slower than equal counts on uneven groups.
 // ---------------------------------------------------------------------------------------------
 constexpr int kMaxGroups = 256;
 struct GroupTable {
     int row_start[kMaxGroups + 1];      // first row of each group in A and a_scale (multiples of 16)
     int out_row_start[kMaxGroups + 1];  // first row of each group in C; the differences are the true row counts
-    int tile_start[kMaxGroups + 1];     // prefix of workgroups
+    int tile_start[kMaxGroups + 1];     // prefix of work items (one per tile); tile_start[groups] is their number
 };
-template <int BM, int BN, int WAVES_M, int WAVES_N>
-__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_grouped(
-    const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
-    const float *__restrict__ SB, uint16_t *__restrict__ C, int M_total, int N, int K, int groups, int tiles_n,
-    int group_m, const GroupTable table) {
-    using G = TileGeom<BM, BN, WAVES_M, WAVES_N>;
-    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
-    // group of this workgroup: the last g with tile_start[g] <= blockIdx.x (empty groups own no workgroup)
+// Work item of this workgroup: its group and its index among the group's items. False: nothing to do (the grid is
+// 8 x the longest piece).
+__device__ __forceinline__ bool grouped_work_item(const GroupTable &table, int groups, int &grp, int &local) {
+    const int xcd = blockIdx.x % NUM_XCD;
+    const long items = table.tile_start[groups];
+    const int item = (int)(items * xcd / NUM_XCD) + (int)(blockIdx.x / NUM_XCD);
+    if (item >= (int)(items * (xcd + 1) / NUM_XCD)) return false;
+    // the last g with tile_start[g] <= item (empty groups own no item)
     int lo = 0, hi = groups;
     while (hi - lo > 1) {
         const int mid = (lo + hi) >> 1;
-        if (table.tile_start[mid] <= (int)blockIdx.x) lo = mid; else hi = mid;
+        if (table.tile_start[mid] <= item) lo = mid; else hi = mid;
     }
-    const int grp = lo, row0 = table.row_start[grp], rows = table.row_start[grp + 1] - row0;
+    grp = lo;
+    local = item - table.tile_start[lo];
+    return true;
+}
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_grouped(
+    const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
+    const float *__restrict__ SB, uint16_t *__restrict__ C, int M_total, int N, int K, int groups,
+    const GroupTable table) {
+    using G = TileGeom<BM, BN, WAVES_M, WAVES_N>;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    int grp, local;
+    if (!grouped_work_item(table, groups, grp, local)) return;
+    const int row0 = table.row_start[grp], rows = table.row_start[grp + 1] - row0;
     const int out0 = table.out_row_start[grp], out_rows = table.out_row_start[grp + 1] - out0;
-    const int local = blockIdx.x - table.tile_start[grp];
     const int tiles_m = (rows + BM - 1) / BM;
-    int tile_m, tile_n;
-    tile_of_block(local, tiles_m * tiles_n, tiles_m, tiles_n, group_m, false, tile_m, tile_n);
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int m0 = (local % tiles_m) * BM, n0 = (local / tiles_m) * BN;
     const int QK = K / BK, QN = (N + 127) / 128;
     f32x4 acc[G::TM][G::TN];
     tile_mainloop<BM, BN, WAVES_M, WAVES_N>(A + row0, B + (size_t)grp * K * N, SA + row0, SB + (size_t)grp * QK * QN,
@@ -873,36 +896,31 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_gro
 
 // The same with two tile heights in one launch: a group's rows are cut into 256-row tiles, and what is left over
 // goes to a 128 x 256 tile when it is at most 128 rows (otherwise to one more 256-row tile). With uneven groups half
-// of the left-overs are that small, and a 128-row tile costs little more than half a 256-row one. tile_start counts
-// a group's workgroups: first its 256-row tiles, then the columns of its 128-row tile. Both paths are 8 waves and
-// share the LDS allocation; the branch is uniform over the workgroup.
+// of the left-overs are that small, and a 128-row tile costs little more than half a 256-row one. A column tile of a
+// group has one work item per row tile, the 128-row one last. Both paths are 8 waves and share the LDS allocation;
+// the branch is uniform over the workgroup.
 __global__ __launch_bounds__(512) void gemm_fp8_blockscale_grouped_mixed(
     const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
-    const float *__restrict__ SB, uint16_t *__restrict__ C, int M_total, int N, int K, int groups, int tiles_n,
-    int group_m, const GroupTable table) {
+    const float *__restrict__ SB, uint16_t *__restrict__ C, int M_total, int N, int K, int groups,
+    const GroupTable table) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
-    int lo = 0, hi = groups;
-    while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (table.tile_start[mid] <= (int)blockIdx.x) lo = mid; else hi = mid;
-    }
-    const int grp = lo, row0 = table.row_start[grp], rows = table.row_start[grp + 1] - row0;
+    int grp, local;
+    if (!grouped_work_item(table, groups, grp, local)) return;
+    const int row0 = table.row_start[grp], rows = table.row_start[grp + 1] - row0;
     const int out0 = table.out_row_start[grp], out_rows = table.out_row_start[grp + 1] - out0;
-    const int local = blockIdx.x - table.tile_start[grp];
     const int big_m = rows / 256 + (rows % 256 > 128 ? 1 : 0);       // 256-row tiles of this group
+    const int tiles_m = rows / 256 + (rows % 256 > 0 ? 1 : 0);       // row tiles of either height
+    const int tile_m = local % tiles_m, n0 = (local / tiles_m) * 256;
     const int QK = K / BK, QN = (N + 127) / 128;
     const uint8_t *Bg = B + (size_t)grp * K * N;
     const float *SBg = SB + (size_t)grp * QK * QN;
-    if (local < big_m * tiles_n) {
-        int tile_m, tile_n;
-        tile_of_block(local, big_m * tiles_n, big_m, tiles_n, group_m, false, tile_m, tile_n);
-        const int m0 = tile_m * 256, n0 = tile_n * 256;
+    if (tile_m < big_m) {
+        const int m0 = tile_m * 256;
         f32x4 acc[TileGeom<256, 256, 2, 4>::TM][TileGeom<256, 256, 2, 4>::TN];
         tile_mainloop<256, 256, 2, 4>(A + row0, Bg, SA + row0, SBg, rows, M_total, N, m0, n0, 0, QK, lds, acc);
         store_tile_bf16<256, 256, 2, 4>(acc, C + (size_t)out0 * N, out_rows, N, m0, n0, lds);
     } else {
         const int r1 = row0 + big_m * 256, rest = rows - big_m * 256;  // 16..128 rows
-        const int n0 = (local - big_m * tiles_n) * 256;
         f32x4 acc[TileGeom<128, 256, 2, 4>::TM][TileGeom<128, 256, 2, 4>::TN];
         tile_mainloop<128, 256, 2, 4>(A + r1, Bg, SA + r1, SBg, rest, M_total, N, 0, n0, 0, QK, lds, acc);
         store_tile_bf16<128, 256, 2, 4>(acc, C + (size_t)(out0 + big_m * 256) * N, out_rows - big_m * 256, N, 0, n0, lds);

@@ -904,7 +904,7 @@ int launch_quantize(const void *x, int rows, int k, void *out, float *scales, hi
 
 namespace {
 typedef void (*grouped_kernel_t)(const uint8_t *, const uint8_t *, const float *, const float *, uint16_t *, int, int, int,
-                                 int, int, int, const rf::GroupTable);
+                                 int, const rf::GroupTable);
 struct GroupedVariant {
     int bm, bn, threads, lds;
     grouped_kernel_t kernel;
@@ -914,6 +914,8 @@ struct GroupedVariant {
         if (!mixed) return ceil_div(rows, bm);
         return rows / 256 + (rows % 256 > 0 ? 1 : 0);
     }
+    // estimated cost of row tile i of a group of `rows` rows, in full-height tiles (the 128-row tile that ends a group
+    // of the mixed form runs 0.6 times as long as a 256-row one), and of all row tiles of one column tile
 };
 #define RF_GROUPED(BM, BN, WM, WN) \
     GroupedVariant { BM, BN, WM *WN * 64, rf::TileGeom<BM, BN, WM, WN>::LDS_BYTES, rf::gemm_fp8_blockscale_grouped<BM, BN, WM, WN>, false }
@@ -1058,8 +1060,9 @@ int grouped_gemm(const void *a, const void *b, const float *as, const float *bs,
         tiles += v.tiles_m(row_offsets[g + 1] - row_offsets[g]) * tiles_n;
     }
     for (int g = groups; g <= rf::kMaxGroups; g++) table.tile_start[g] = tiles;
-    hipLaunchKernelGGL(v.kernel, dim3(tiles), dim3(v.threads), v.lds, stream, (const uint8_t *)a, (const uint8_t *)b, as,
-                       bs, (uint16_t *)c, m_rows, n, k, groups, tiles_n, 8, table);
+    const int longest = ceil_div(tiles, rf::NUM_XCD);          // every XCD takes an eighth of the tiles, rounded
+    hipLaunchKernelGGL(v.kernel, dim3(longest * rf::NUM_XCD), dim3(v.threads), v.lds, stream, (const uint8_t *)a,
+                       (const uint8_t *)b, as, bs, (uint16_t *)c, m_rows, n, k, groups, table);
     RF_HIP(hipGetLastError());
     return RF_OK;
 }
