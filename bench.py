@@ -429,11 +429,16 @@ def main():
             u = e0.elapsed_time(e1) * 1e3 / 50
             tf = 2.0 * gm * gn * gk / u / 1e6
             sizes = [b - a for a, b in zip(offs_, offs_[1:])]
+            # every expert's weights are read once: with 256 rows per expert on average they are most of the bytes
+            gbytes = gm * gk + gg * gn * gk + 2 * gm * gn + 4 * (gk // 128) * (gm + gg * (gn // 128))
             out[key] = {"workload": "32 groups, %d rows in total (%d..%d per group), N=%d K=%d" % (
                             gm, min(sizes), max(sizes), gn, gk),
-                        "us": round(u, 2), "tflops": round(tf, 1), "pct_fp8_mfma_peak": round(100 * tf / PEAK_FP8_TFLOPS, 2)}
-            print("%s %s: %.2f us  %.1f TFLOP/s (%.1f %% of peak)" % (key, out[key]["workload"], u, tf,
-                  100 * tf / PEAK_FP8_TFLOPS), file=sys.stderr)
+                        "us": round(u, 2), "tflops": round(tf, 1), "pct_fp8_mfma_peak": round(100 * tf / PEAK_FP8_TFLOPS, 2),
+                        "algorithmic_mb": round(gbytes / 1e6, 1), "gbs": round(gbytes / u / 1e3, 1),
+                        "pct_hbm_peak": round(100 * gbytes / u / 1e3 / PEAK_HBM_GBS, 2)}
+            print("%s %s: %.2f us  %.1f TFLOP/s (%.1f %% of the fp8 peak), %.0f GB/s algorithmic (%.1f %% of 8 TB/s)" % (
+                  key, out[key]["workload"], u, tf, 100 * tf / PEAK_FP8_TFLOPS, gbytes / u / 1e3,
+                  100 * gbytes / u / 1e3 / PEAK_HBM_GBS), file=sys.stderr)
         # arbitrary sizes again, with the activations quantised straight into the padded layout (quantize_a_grouped):
         # no staging copy at all
         offs_any = [0] + [int(x) for x in cuts_any] + [8192]
