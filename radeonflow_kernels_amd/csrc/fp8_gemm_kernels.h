@@ -484,11 +484,13 @@ __device__ __forceinline__ void tile_mainloop(
 }
 
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-// 16 bytes of C. The store carries device scope (sc1): the line is written through to memory instead of staying dirty
-// in the XCD's L2 until the end of the kernel. C is written once and not read again, and with 56 to 88 MB of it the
-// write-back at the end of the kernel was time that nothing overlapped (6144 x 7168 x 2048: 89.4 -> 87.2 us;
-// non-temporal hints measured slower than either).
-__device__ __forceinline__ void store_c16(uint16_t *p, const uint4 &v) {
+// 16 bytes of C or of a split-K partial sum. The store carries device scope (sc1): the line is written through to
+// memory instead of staying dirty in the XCD's L2 until the end of the kernel. C is written once and not read again,
+// and with 56 to 88 MB of it the write-back at the end of the kernel was time that nothing overlapped (6144 x 7168 x
+// 2048: 89.4 -> 87.2 us; non-temporal hints measured slower than either). The fp32 partial sums of a K split are read
+// next by the reduction kernel, on whatever XCD its workgroups land, so they have to leave this L2 anyway
+// (1024 x 1536 x 7168 with 4 splits: 24.2 -> 23.5 us, 1024 x 576 x 7168 with 8: 17.9 -> 17.0 us).
+__device__ __forceinline__ void store_c16(void *p, const uint4 &v) {
     const u32x4 w = {v.x, v.y, v.z, v.w};
     // A store of more than 8 bytes reads its data registers a little after it has been issued; the compiler keeps
     // vector instructions that overwrite them away from its own stores, but it does not look inside this statement.
@@ -648,7 +650,7 @@ __device__ __forceinline__ void store_tile_f32_staged(const f32x4 (&acc)[BM / WA
                 const int r = r0 + lane / LPR, cb = (lane % LPR) * 16;
                 const uint4 v = *(const uint4 *)(region + r * ROW + cb);
                 const int m = wm * G::WM + 16 * j + r, n = wn * G::WN + cb / 4;
-                if (m < m_lim && n < n_lim) *(uint4 *)(t + (size_t)m * ld + n) = v;
+                if (m < m_lim && n < n_lim) store_c16(t + (size_t)m * ld + n, v);
             }
         } else {
             // rows of LPR chunks with 64 % LPR != 0: the m-tile's chunks in row-major order, 64 per instruction
@@ -657,7 +659,7 @@ __device__ __forceinline__ void store_tile_f32_staged(const f32x4 (&acc)[BM / WA
                 const int q = q0 + lane, r = q / LPR, cb = (q % LPR) * 16;
                 const uint4 v = *(const uint4 *)(region + r * ROW + cb);
                 const int m = wm * G::WM + 16 * j + r, n = wn * G::WN + cb / 4;
-                if (m < m_lim && n < n_lim) *(uint4 *)(t + (size_t)m * ld + n) = v;
+                if (m < m_lim && n < n_lim) store_c16(t + (size_t)m * ld + n, v);
             }
         }
     }
