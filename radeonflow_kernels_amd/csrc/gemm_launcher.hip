@@ -362,7 +362,7 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
         return;
     }
     // No measured entry: a cost model fitted to the tuner's measurements of the tabled shapes (on those
-    // 111 shapes its plan is 1 % slower than the best measured one on average, 12 % at worst). Time in microseconds of a plan =
+    // 103 shapes its plan is 1 % slower than the best measured one on average, 8 % at worst). Time in microseconds of a plan =
     //   rounds * (K blocks per workgroup * c + f)           one workgroup per tile and K split
     //   rounds * K blocks * c + f + (rounds - 1) * f_next   persistent: only the first tile starts cold
     //   + reduction cost when K is split
@@ -371,8 +371,8 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
     // the 64x128 tile where M is short or the whole problem is a few microseconds); the others never won by more than
     // a few percent.
     struct Candidate { int variant; double c, f; };
-    const Candidate cands[] = {{0, 1.055, 7.96}, {3, 0.709, 4.81}, {5, 0.71, 5.2}, {6, 0.65, 4.0}, {7, 0.79, 0.0}};
-    const double f_next = 3.0, reduce_fixed = 6.43, reduce_per_elem = 1.07e-6;
+    const Candidate cands[] = {{0, 1.055, 7.46}, {3, 0.619, 5.11}, {5, 0.71, 5.2}, {6, 0.68, 4.3}, {7, 0.85, 0.0}};
+    const double f_next = 3.3, reduce_fixed = 4.83, reduce_per_elem = 1.07e-6;
     const int splits_tried[] = {1, 2, 3, 4, 6, 8, 12, 16};
     const int qk = k / rf::BK;
     double best_cost = 1e30;
