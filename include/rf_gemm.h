@@ -58,8 +58,8 @@ typedef struct rf_gemm_config {
                          1 STREAM_K   persistent grid, one workgroup per CU, equal shares of the tile x K-block work
                                       line; needs split_k == 1 and at least as many tiles as CUs;
                          2 PERSISTENT persistent grid, whole tiles, one load/compute pipeline running across the
-                                      tiles of a workgroup; needs split_k == 1, M and N multiples of the tile,
-                                      K/128 even */
+                                      tiles of a workgroup; needs split_k == 1, M a multiple of 16 and at least the
+                                      tile height, N a multiple of the tile width, K/128 even */
 } rf_gemm_config;
 
 /* Drop-in for the reference's launcher entry (src/gemm/gemm_launcher.cpp:182-184):

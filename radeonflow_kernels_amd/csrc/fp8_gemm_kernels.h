@@ -583,9 +583,12 @@ __device__ __forceinline__ void store_tile_bf16(const f32x4 (&acc)[BM / WAVES_M 
 // load) and keeps them in order with the reads.
 typedef uint32_t staged_u32x2 __attribute__((ext_vector_type(2), may_alias));
 typedef uint32_t staged_u32x4 __attribute__((ext_vector_type(4), may_alias));
-template <int BM, int BN, int WAVES_M, int WAVES_N>
+// MASKED: only the tile's first row_lim rows exist in C (a caller whose M is not a multiple of 16 has padded A and
+// a_scale, not C); whole columns always.
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool MASKED = false>
 __device__ __forceinline__ void store_whole_tile_bf16(const f32x4 (&acc)[BM / WAVES_M / 16][BN / WAVES_N / 16],
-                                                      uint16_t *__restrict__ C, int N, int m0, int n0, uint8_t *staging) {
+                                                      uint16_t *__restrict__ C, int N, int m0, int n0, uint8_t *staging,
+                                                      int row_lim = BM) {
     using G = TileGeom<BM, BN, WAVES_M, WAVES_N>;
     constexpr int ROW = G::WN * 2 + 16;                  // bytes per staged row
     constexpr int LPR = G::WN * 2 / 16;                  // lanes per row on the way out (16 bytes each)
@@ -614,7 +617,8 @@ __device__ __forceinline__ void store_whole_tile_bf16(const f32x4 (&acc)[BM / WA
 #pragma unroll
             for (int q = 0; q < NI; q++) {
                 const staged_u32x4 x = v[(j - 1) & 1][q];
-                store_c16(out + (size_t)((j - 1) * 16 + q * RPI) * N, make_uint4(x[0], x[1], x[2], x[3]));
+                if (!MASKED || wm * G::WM + (j - 1) * 16 + q * RPI + lane / LPR < row_lim)
+                    store_c16(out + (size_t)((j - 1) * 16 + q * RPI) * N, make_uint4(x[0], x[1], x[2], x[3]));
             }
         }
     }

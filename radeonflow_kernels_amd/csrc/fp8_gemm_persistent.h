@@ -8,9 +8,13 @@
 // the bf16 store of the finished tile runs from a private LDS region while the next stage is already resident.
 // Tiles with few K blocks (K = 256: two per tile) gain the most.
 //
-// Restrictions (checked by the host): M % BM == 0 and N % BN == 0 (per-lane load offsets are tile-independent, the
-// tile origin lives in the scalar base pointers), K/128 even (a tile starts on LDS stage 0). Numerics and the
-// per-tile instruction schedule are those of tile_mainloop.
+// Restrictions (checked by the host): M >= BM, M % 16 == 0 and N % BN == 0 (per-lane load offsets are
+// tile-independent, the tile origin lives in the scalar base pointers: every tile is a whole tile), K/128 even (a
+// tile starts on LDS stage 0). When M is not a multiple of BM the last row of tiles starts at row M - BM instead of
+// tiles_m * BM - BM: it overlaps the row of tiles before it, both compute the rows they share from the same operands
+// with the same instructions and store the same values. M_store <= M is the number of rows of C that exist (a caller
+// whose M is not a multiple of 16 passes A and a_scale padded to M rows and its own C). Numerics and the per-tile
+// instruction schedule are those of tile_mainloop.
 #pragma once
 #include "fp8_gemm_kernels.h"
 
@@ -30,7 +34,7 @@ template <int BM, int BN, int WAVES_M, int WAVES_N>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_persistent(
     const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
     const float *__restrict__ SB, uint16_t *__restrict__ C, int M, int N, int K, int tiles_m, int tiles_n,
-    int group_m) {
+    int group_m, int M_store) {
     using G = TileGeom<BM, BN, WAVES_M, WAVES_N>;
     using P = PersistentGeom<BM, BN, WAVES_M, WAVES_N>;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
@@ -65,7 +69,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
         int tm, tn;
         const int r = lane < my_tiles - 1 ? lane : my_tiles - 1;
         tile_of_block(blockIdx.x + r * gridDim.x, T, tiles_m, tiles_n, group_m, true, tm, tn);
-        m0_of_lane = tm * BM;
+        m0_of_lane = tm * BM < M - BM ? tm * BM : M - BM;
         n0_of_lane = tn * BN;
     }
     auto tile_origin = [&](int r, int &m0, int &n0) {
@@ -76,7 +80,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
         } else {
             int tm, tn;
             tile_of_block(blockIdx.x + r * gridDim.x, T, tiles_m, tiles_n, group_m, true, tm, tn);
-            m0 = __builtin_amdgcn_readfirstlane(tm * BM);
+            m0 = __builtin_amdgcn_readfirstlane(tm * BM < M - BM ? tm * BM : M - BM);
             n0 = __builtin_amdgcn_readfirstlane(tn * BN);
         }
     };
@@ -327,7 +331,11 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
         // the next tile (with two K blocks per tile: 0.7 us of each tile's 4.4).
 #pragma unroll
         for (int d = TN; d < NDMA; d++) issue_dma(d, 1, dsrc[d]);
-        store_whole_tile_bf16<BM, BN, WAVES_M, WAVES_N>(acc, C, N, m0_cur, n0_cur, lds + P::STAGING_OFF);
+        if (m0_cur + BM <= M_store)
+            store_whole_tile_bf16<BM, BN, WAVES_M, WAVES_N>(acc, C, N, m0_cur, n0_cur, lds + P::STAGING_OFF);
+        else                                              // the last rows of A are padding: C does not have them
+            store_whole_tile_bf16<BM, BN, WAVES_M, WAVES_N, true>(acc, C, N, m0_cur, n0_cur, lds + P::STAGING_OFF,
+                                                                  M_store - m0_cur);
 #pragma unroll
         for (int j = 0; j < TM; j++)
 #pragma unroll

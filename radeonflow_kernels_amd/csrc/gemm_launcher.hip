@@ -45,7 +45,7 @@ typedef void (*tile_kernel_t)(const uint8_t *, const uint8_t *, const float *, c
 typedef void (*streamk_kernel_t)(const uint8_t *, const uint8_t *, const float *, const float *, uint16_t *, int, int,
                                  int, int, int, int, unsigned *, float *);
 typedef void (*persistent_kernel_t)(const uint8_t *, const uint8_t *, const float *, const float *, uint16_t *, int, int,
-                                    int, int, int, int);
+                                    int, int, int, int, int);
 struct Variant {
     int bm, bn, waves_m, waves_n, lds;
     tile_kernel_t direct, partial;
@@ -316,7 +316,7 @@ bool tiled_path_ok(const void *a, const void *b, const void *c, int m, int n) {
 }
 
 bool persistent_ok(const Variant &v, int m, int n, int k) {
-    return v.persistent && m % v.bm == 0 && n % v.bn == 0 && (k / rf::BK) % 2 == 0;
+    return v.persistent && m >= v.bm && m % 16 == 0 && n % v.bn == 0 && (k / rf::BK) % 2 == 0;
 }
 
 // Stream-K: at least one tile per workgroup (then a split tile has exactly two contributors, which is all the kernel
@@ -420,7 +420,7 @@ int launch_locked(State &s, Mem &mem, const void *a, const void *b, const float 
                 return fail(RF_ERR_BAD_CONFIG, "stream_k needs at least as many tiles as compute units");
         } else if (cfg.stream_k == RF_SCHEDULE_PERSISTENT) {
             if (!persistent_ok(kVariants[cfg.variant], m, n, k))
-                return fail(RF_ERR_BAD_CONFIG, "the persistent schedule needs M, N multiples of the tile and K/128 even");
+                return fail(RF_ERR_BAD_CONFIG, "the persistent schedule needs M >= the tile height, M % 16 == 0, N a multiple of the tile width and K/128 even");
         } else if (cfg.stream_k != RF_SCHEDULE_TILES) {
             return fail(RF_ERR_BAD_CONFIG, "unknown schedule");
         }
@@ -428,7 +428,7 @@ int launch_locked(State &s, Mem &mem, const void *a, const void *b, const float 
         select_config(m, n, k, s.num_cu, tiled_ok, shared().user_plans, &cfg);
     }
 
-    if (m_store != m && (cfg.variant < 0 || cfg.stream_k != RF_SCHEDULE_TILES))
+    if (m_store != m && (cfg.variant < 0 || cfg.stream_k == RF_SCHEDULE_STREAM_K))
         return fail(RF_ERR_BAD_CONFIG, "internal: this schedule cannot write fewer rows than it computes");
     if (cfg.variant < 0) {
         dim3 grid(ceil_div(n, 16), ceil_div(m, 16));
@@ -454,7 +454,7 @@ int launch_locked(State &s, Mem &mem, const void *a, const void *b, const float 
         const int P = s.num_cu * (per_cu < 1 ? 1 : per_cu);
         hipLaunchKernelGGL(v.persistent, dim3(T < P ? T : P), block, v.lds_persistent, stream,
                            (const uint8_t *)a, (const uint8_t *)b, as, bs, (uint16_t *)c, m, n, k, tiles_m, tiles_n,
-                           cfg.group_m);
+                           cfg.group_m, m_store);
         RF_HIP(hipGetLastError());
         return RF_OK;
     }
@@ -625,11 +625,12 @@ int launch_padded(State &s, Mem &mem, const void *a, const void *b, const float 
     const int mp = pad16(m), np = pad16(n), qk = k / rf::BK;
     const bool copy_a = mp != m || (uintptr_t)a % 16 != 0, copy_b = np != n || (uintptr_t)b % 16 != 0;
     const bool copy_sa = mp != m;
-    // The plan of the padded shape. With whole columns and an aligned c, a plan of one workgroup per tile writes the m
-    // true rows straight into c (its stores are masked by row); otherwise C is staged and copied back.
+    // The plan of the padded shape. With whole columns and an aligned c, the whole-tile schedules (one workgroup per
+    // tile, persistent) write the m true rows straight into c (their stores are masked by row); otherwise C is staged
+    // and copied back.
     rf_gemm_config cfg;
     select_config(mp, np, k, s.num_cu, true, shared().user_plans, &cfg);
-    const bool copy_c = np != n || (uintptr_t)c % 16 != 0 || (mp != m && cfg.stream_k != RF_SCHEDULE_TILES);
+    const bool copy_c = np != n || (uintptr_t)c % 16 != 0 || (mp != m && cfg.stream_k == RF_SCHEDULE_STREAM_K);
     size_t off = 0;
     const size_t off_a = off;  off += copy_a ? align((size_t)k * mp) : 0;
     const size_t off_b = off;  off += copy_b ? align((size_t)k * np) : 0;

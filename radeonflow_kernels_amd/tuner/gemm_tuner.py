@@ -81,7 +81,7 @@ def tune_shape(rfk, m, n, k, log=print):
         for split, sk in [(sp, 0) for sp in SPLITS] + [(1, 1), (1, 2)]:
             if split > k // 128 or (sk == 1 and (tiles < ncu or not v["stream_k"])):
                 continue
-            if sk == 2 and (not v["persistent"] or m % v["block_m"] or n % v["block_n"] or (k // 128) % 2):
+            if sk == 2 and (not v["persistent"] or m < v["block_m"] or m % 16 or n % v["block_n"] or (k // 128) % 2):
                 continue
             for gm in GROUPS:
                 cfg = rfk.GemmConfig(v["variant"], split, gm, sk)

@@ -148,6 +148,49 @@ def test_persistent_schedule_bit_exact(rfk, m, n, k):
     assert tried > 0
 
 
+@pytest.mark.parametrize("m,n,k", [(272, 512, 256), (624, 768, 512), (1008, 1024, 256), (2000, 512, 768)])
+def test_persistent_schedule_with_a_last_row_of_tiles_that_overlaps_the_one_before(rfk, m, n, k):
+    """M is a multiple of 16 but not of the tile height: the last row of tiles starts at M - BM and shares rows with
+    its neighbour. Exact data against the oracle, bit for bit, twice; then data with rounding in it against the
+    one-workgroup-per-tile kernel of the same variant, bit for bit as well and the same on every launch: a row's result
+    does not depend on where in a tile the row sits, so both tiles that compute a shared row store the same value."""
+    data = exact_problem(m, n, k, seed=3 * m + n + k)
+    exp = oracle_bf16(data)
+    noisy = rk.generate_input_blockquant(m, n, k, seed=m + k)
+    tried = 0
+    for v in rfk.variants():
+        if not v["persistent"] or m < v["block_m"] or m % v["block_m"] == 0 or n % v["block_n"]:
+            continue
+        cfg = rfk.GemmConfig(v["variant"], 1, 8, 2)
+        for rep in range(2):
+            out = _run(rfk, data, config=cfg, canary=1024)
+            assert np.array_equal(bf16_bits(out), exp), "plan %r rep %d" % (cfg, rep)
+        tiles = bf16_bits(_run(rfk, noisy, config=rfk.GemmConfig(v["variant"], 1, 8, 0), canary=1024)).copy()
+        for rep in range(3):
+            out = _run(rfk, noisy, config=cfg, canary=1024)
+            assert np.array_equal(bf16_bits(out), tiles), "plan %r rep %d differs from the tile kernel" % (cfg, rep)
+        tried += 1
+    assert tried > 0
+
+
+def test_ragged_m_under_a_persistent_plan_writes_c_in_place(rfk, tmp_path):
+    """M = 1001: A and a_scale are staged with 1008 rows; with a persistent plan for the padded shape the kernel writes
+    the 1001 true rows straight into C (the last tile's stores are masked by row) and nothing behind them."""
+    m, n, k = 1001, 1024, 512
+    path = tmp_path / "p.plans"
+    path.write_text("1008 %d %d 0 1 8 2\n" % (n, k))
+    data = exact_problem(m, n, k, seed=77)
+    try:
+        assert rfk.load_plans(str(path)) == 1
+        got = rfk.select_config(1008, n, k)
+        assert (got.variant, got.stream_k) == (0, 2)
+        for rep in range(2):
+            out = _run(rfk, data, canary=2048)
+            assert np.array_equal(bf16_bits(out), oracle_bf16(data)), "rep %d" % rep
+    finally:
+        rfk.clear_plans()
+
+
 def test_persistent_schedule_rejects_ragged_shapes(rfk):
     data = exact_problem(272, 144, 256, seed=1)
     with pytest.raises(RuntimeError):
@@ -280,14 +323,14 @@ def test_plans_loaded_from_a_file_take_precedence_and_can_be_cleared(rfk, tmp_pa
     other = rfk.select_config(1024, 1536, 7168)
     forced = (1, 2, 4, 0) if (before.variant, before.split_k) != (1, 2) else (3, 1, 4, 0)
     path = tmp_path / "my.plans"
-    path.write_text("%d %d %d 0 1 8 2\n" % (m + 16, n, k)                       # persistent on a ragged shape: skipped
+    path.write_text("%d %d %d 0 1 8 2\n" % (m, n, k + 128)                      # persistent with an odd number of K blocks: skipped
                     + "%d %d %d %d %d %d %d\n" % ((m, n, k) + forced))
     try:
         assert rfk.load_plans(str(path)) == 2
         got = rfk.select_config(m, n, k)
         assert (got.variant, got.split_k, got.group_m, got.stream_k) == forced
-        ragged = rfk.select_config(m + 16, n, k)
-        assert ragged.stream_k != 2
+        odd = rfk.select_config(m, n, k + 128)
+        assert odd.stream_k != 2
         again = rfk.select_config(1024, 1536, 7168)
         assert (again.variant, again.split_k, again.stream_k) == (other.variant, other.split_k, other.stream_k)
         data = exact_problem(m, n, k, seed=77)
