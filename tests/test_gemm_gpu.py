@@ -191,6 +191,17 @@ def test_ragged_m_under_a_persistent_plan_writes_c_in_place(rfk, tmp_path):
         rfk.clear_plans()
 
 
+@pytest.mark.parametrize("m", [6000, 6001])
+def test_large_m_that_is_not_a_tile_multiple_runs_the_persistent_plan_automatically(rfk, m):
+    """6000 and 6001 rows with C4's N and K: the automatic plan is the persistent schedule (for 6001 on the shape padded
+    to 6016 rows, with C written in place); exact data, bit for bit, canary behind the last true row intact."""
+    n, k = 7168, 256
+    assert rfk.select_config(m, n, k).stream_k == 2
+    data = exact_problem(m, n, k, seed=m)
+    out = _run(rfk, data, canary=8192)
+    assert np.array_equal(bf16_bits(out), oracle_bf16(data))
+
+
 def test_persistent_schedule_rejects_ragged_shapes(rfk):
     data = exact_problem(272, 144, 256, seed=1)
     with pytest.raises(RuntimeError):
