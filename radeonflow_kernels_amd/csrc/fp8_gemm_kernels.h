@@ -133,7 +133,7 @@ __device__ __forceinline__ void tile_mainloop(
     // of any stage is "per-lane base register + immediate": no address arithmetic in the loop.
     constexpr int STAGE_A = G::STAGE_A, STAGE_B = G::STAGE_B, STAGE_S = G::STAGE_S;
     constexpr int OFF_B = NS * STAGE_A, OFF_S = NS * (STAGE_A + STAGE_B), OFF_SB = BM * 4;   // OFF_SB inside an S region
-    static_assert(NS == 2, "more than two stages would need vmcnt(n > 0) waits, which LDS-DMA loads do not support safely");
+    static_assert(NS == 2 || NS == 3, "two stages (one K block in flight) or three (two in flight)");
     constexpr int INST_A = STAGE_A / 1024 / NW, INST_B = STAGE_B / 1024 / NW;   // 1 KiB per wave instruction
     constexpr int NSC = BM / 64;                                                // scale loads: 64 floats each
     static_assert(STAGE_A % (1024 * NW) == 0 && STAGE_B % (1024 * NW) == 0, "loads must divide evenly over waves");
@@ -261,10 +261,14 @@ __device__ __forceinline__ void tile_mainloop(
                          :: "v"(goff_sb), "s"(src), "s"(lds_dst_sb), "n"(stage * STAGE_S) : "memory", "scc");
         }
     };
-    // Wait until every load this wave has issued has landed. Only vmcnt(0) is used: with LDS-DMA loads a wait for
-    // "all but the newest n" is not safe (a later load that hits in L2 was seen to complete before an earlier one
-    // that missed), which is also why the kernel has exactly two stages.
-    auto wait_for_stage = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
+    // Wait until the loads of the stage that is read next have landed. Two stages: every load this wave has issued.
+    // Three stages: all but the loads of the newest block; a wave's loads complete in the order it issued them, every
+    // wave issues at least INST_A + INST_B per block (those with scale loads one or two more, whose oldest then have
+    // to land as well), so "all but the newest INST_A + INST_B" covers it.
+    auto wait_for_stage = [&]() {
+        if constexpr (NS == 2) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(%0)" :: "n"(INST_A + INST_B) : "memory");
+    };
 
     // ---- LDS -> MFMA operands: per-lane byte offsets of the transpose reads (stage 0, t = 0) ----
     // lane (L,g) of read t points at row k = 32g + 8t + L/2, half (L&1) of 16-byte chunk c.
@@ -458,11 +462,21 @@ __device__ __forceinline__ void tile_mainloop(
     auto k_loop = [&](auto split_c) {
         constexpr int split = decltype(split_c)::value;
         int kb = kb_begin;
-        for (; kb + 1 < kb_end; kb += 2) {
-            k_block(IntTag<0>{}, split_c, kb);
-            k_block(IntTag<1>{}, split_c, kb + 1);
+        if constexpr (NS == 2) {
+            for (; kb + 1 < kb_end; kb += 2) {
+                k_block(IntTag<0>{}, split_c, kb);
+                k_block(IntTag<1>{}, split_c, kb + 1);
+            }
+            if (kb < kb_end) k_block(IntTag<0>{}, split_c, kb);
+        } else {
+            for (; kb + 2 < kb_end; kb += 3) {
+                k_block(IntTag<0>{}, split_c, kb);
+                k_block(IntTag<1>{}, split_c, kb + 1);
+                k_block(IntTag<2>{}, split_c, kb + 2);
+            }
+            if (kb < kb_end) k_block(IntTag<0>{}, split_c, kb);
+            if (kb + 1 < kb_end) k_block(IntTag<1>{}, split_c, kb + 1);
         }
-        if (kb < kb_end) k_block(IntTag<0>{}, split_c, kb);
         // folds still owed by the last K block
 #pragma unroll
         for (int t = 0; t < LAG; t++) {
@@ -711,7 +725,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
     const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
     const float *__restrict__ SB, void *__restrict__ Cout, int M, int N, int K, int kb_per_split,
     int tiles_m, int tiles_n, int group_m, int M_store) {
-    using G = TileGeom<BM, BN, WAVES_M, WAVES_N>;
+    using G = TileGeom<BM, BN, WAVES_M, WAVES_N, NS>;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     int tile_m, tile_n;
     tile_of_block(blockIdx.x, tiles_m * tiles_n, tiles_m, tiles_n, group_m, true, tile_m, tile_n);
@@ -880,7 +894,7 @@ __device__ __forceinline__ bool grouped_work_item(const GroupTable &table, int g
     local = item - table.tile_start[lo];
     return true;
 }
-template <int BM, int BN, int WAVES_M, int WAVES_N>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NS = 2>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_grouped(
     const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
     const float *__restrict__ SB, uint16_t *__restrict__ C, int M_total, int N, int K, int groups,
@@ -895,8 +909,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_gro
     const int m0 = (local % tiles_m) * BM, n0 = (local / tiles_m) * BN;
     const int QK = K / BK, QN = (N + 127) / 128;
     f32x4 acc[G::TM][G::TN];
-    tile_mainloop<BM, BN, WAVES_M, WAVES_N>(A + row0, B + (size_t)grp * K * N, SA + row0, SB + (size_t)grp * QK * QN,
-                                            rows, M_total, N, m0, n0, 0, QK, lds, acc);
+    tile_mainloop<BM, BN, WAVES_M, WAVES_N, NS>(A + row0, B + (size_t)grp * K * N, SA + row0,
+                                                SB + (size_t)grp * QK * QN, rows, M_total, N, m0, n0, 0, QK, lds, acc);
     store_tile_bf16<BM, BN, WAVES_M, WAVES_N>(acc, C + (size_t)out0 * N, out_rows, N, m0, n0, lds);
 }
 
@@ -928,7 +942,7 @@ __global__ __launch_bounds__(512) void gemm_fp8_blockscale_grouped_mixed(
     } else {
         const int r1 = row0 + big_m * 256, rest = rows - big_m * 256;  // 16..128 rows
         f32x4 acc[TileGeom<128, 256, 2, 4>::TM][TileGeom<128, 256, 2, 4>::TN];
-        tile_mainloop<128, 256, 2, 4>(A + r1, Bg, SA + r1, SBg, rest, M_total, N, 0, n0, 0, QK, lds, acc);
+        tile_mainloop<128, 256, 2, 4, 3>(A + r1, Bg, SA + r1, SBg, rest, M_total, N, 0, n0, 0, QK, lds, acc);
         store_tile_bf16<128, 256, 2, 4>(acc, C + (size_t)(out0 + big_m * 256) * N, out_rows - big_m * 256, N, 0, n0, lds);
     }
 }

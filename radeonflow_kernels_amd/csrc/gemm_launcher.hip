@@ -67,6 +67,15 @@ struct Variant {
     Variant { BM, BN, WM, WN, rf::TileGeom<BM, BN, WM, WN>::LDS_BYTES,                     \
               rf::gemm_fp8_blockscale_tile<BM, BN, WM, WN, false>,                         \
               rf::gemm_fp8_blockscale_tile<BM, BN, WM, WN, true>, nullptr, nullptr, 0 }
+// the same with three LDS stages: two K blocks in flight instead of one. A K block of these tiles is 0.4 us of MFMAs,
+// less than a load takes to come back from L2 or the Infinity Cache on a busy chip, so with two stages the loop ran at
+// the latency of its loads: 1024 x 4608 x 7168 45.6 -> 39.0 us, 256 x 7168 x 2304 15.6 -> 13.1 us; the best plan of 54
+// of the 103 tabled shapes. The two-stage forms stay: they fit more workgroups per CU (64 x 128: three instead of
+// two), which the smallest problems prefer. (128 x 128 with three stages never won and is not built.)
+#define RF_VARIANT_TILE_ONLY_NS3(BM, BN, WM, WN)                                           \
+    Variant { BM, BN, WM, WN, rf::TileGeom<BM, BN, WM, WN, 3>::LDS_BYTES,                  \
+              rf::gemm_fp8_blockscale_tile<BM, BN, WM, WN, false, 3>,                      \
+              rf::gemm_fp8_blockscale_tile<BM, BN, WM, WN, true, 3>, nullptr, nullptr, 0 }
 const Variant kVariants[] = {
     RF_VARIANT(256, 256, 2, 4),   // 0: 8 waves, wave tile 128(m) x 64(n), 128 KiB LDS
     RF_VARIANT(128, 128, 2, 2),   // 1: 4 waves, wave tile 64 x 64, 64 KiB LDS (2 workgroups per CU)
@@ -76,6 +85,10 @@ const Variant kVariants[] = {
     RF_VARIANT_TILE_ONLY(192, 192, 2, 4),   // 5: 8 waves, wave tile 96 x 48, 98 KiB LDS (6144 x 4608 = 768 tiles = 3 x 256)
     RF_VARIANT_TILE_ONLY(128, 192, 2, 4),   // 6: 8 waves, wave tile 64 x 48, 82 KiB LDS (N = 576, 1536: no padded columns)
     RF_VARIANT_TILE_ONLY(64, 128, 2, 2),    // 7: 4 waves, wave tile 32 x 64, 49 KiB LDS (3 workgroups per CU; short M)
+    RF_VARIANT_TILE_ONLY_NS3(128, 192, 2, 4),   // 8: variant 6 with three stages, 123 KiB LDS
+    RF_VARIANT_TILE_ONLY_NS3(64, 128, 2, 2),    // 9: variant 7 with three stages, 74 KiB LDS (2 workgroups per CU)
+    RF_VARIANT_TILE_ONLY_NS3(128, 256, 2, 4),   // 10: variant 3 with three stages, 149 KiB LDS
+    RF_VARIANT_TILE_ONLY_NS3(192, 192, 2, 4),   // 11: variant 5 with three stages, 147 KiB LDS
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
@@ -362,17 +375,18 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
         return;
     }
     // No measured entry: a cost model fitted to the tuner's measurements of the tabled shapes (on those
-    // 103 shapes its plan is 1 % slower than the best measured one on average, 8 % at worst). Time in microseconds of a plan =
+    // 103 shapes its plan is 0.8 % slower than the best measured one on average, 8 % at worst). Time in microseconds of a plan =
     //   rounds * (K blocks per workgroup * c + f)           one workgroup per tile and K split
     //   rounds * K blocks * c + f + (rounds - 1) * f_next   persistent: only the first tile starts cold
     //   + reduction cost when K is split
-    // with rounds = ceil(workgroups / CUs). Candidates: the 256x256, 128x256, 192x192, 128x192 and 64x128 tiles (192-wide
-    // tiles win where they divide the shape into fuller rounds or leave no padded columns, e.g. N = 576, 1536 or 3072;
-    // the 64x128 tile where M is short or the whole problem is a few microseconds); the others never won by more than
-    // a few percent.
+    // with rounds = ceil(workgroups / CUs). Candidates: the 256x256 tile and the 128x256, 192x192, 128x192 and 64x128
+    // tiles with two and with three stages (192-wide tiles win where they divide the shape into fuller rounds or leave
+    // no padded columns, e.g. N = 576, 1536 or 3072; the 64x128 tile where M is short or the whole problem is a few
+    // microseconds); the others never won by more than a few percent.
     struct Candidate { int variant; double c, f; };
-    const Candidate cands[] = {{0, 1.055, 7.46}, {3, 0.619, 5.11}, {5, 0.71, 5.2}, {6, 0.68, 4.3}, {7, 0.85, 0.0}};
-    const double f_next = 3.3, reduce_fixed = 4.83, reduce_per_elem = 1.07e-6;
+    const Candidate cands[] = {{0, 0.955, 7.96}, {3, 0.619, 5.11}, {5, 0.71, 5.2},  {6, 0.74, 3.7},  {7, 0.82, 0.0},
+                               {8, 0.52, 4.5},   {9, 0.70, 0.5},   {10, 0.53, 5.9}, {11, 0.62, 5.8}};
+    const double f_next = 3.0, reduce_fixed = 2.83, reduce_per_elem = 1.37e-6;
     const int splits_tried[] = {1, 2, 3, 4, 6, 8, 12, 16};
     const int qk = k / rf::BK;
     double best_cost = 1e30;
@@ -918,11 +932,13 @@ struct GroupedVariant {
     // estimated cost of row tile i of a group of `rows` rows, in full-height tiles (the 128-row tile that ends a group
     // of the mixed form runs 0.6 times as long as a 256-row one), and of all row tiles of one column tile
 };
-#define RF_GROUPED(BM, BN, WM, WN) \
-    GroupedVariant { BM, BN, WM *WN * 64, rf::TileGeom<BM, BN, WM, WN>::LDS_BYTES, rf::gemm_fp8_blockscale_grouped<BM, BN, WM, WN>, false }
+#define RF_GROUPED(BM, BN, WM, WN, NS) \
+    GroupedVariant { BM, BN, WM *WN * 64, rf::TileGeom<BM, BN, WM, WN, NS>::LDS_BYTES, rf::gemm_fp8_blockscale_grouped<BM, BN, WM, WN, NS>, false }
+constexpr int kMixedLds = rf::TileGeom<256, 256, 2, 4>::LDS_BYTES > rf::TileGeom<128, 256, 2, 4, 3>::LDS_BYTES
+                              ? rf::TileGeom<256, 256, 2, 4>::LDS_BYTES : rf::TileGeom<128, 256, 2, 4, 3>::LDS_BYTES;
 const GroupedVariant kGroupedVariants[] = {
-    RF_GROUPED(256, 256, 2, 4), RF_GROUPED(128, 256, 2, 4), RF_GROUPED(128, 128, 2, 2), RF_GROUPED(128, 64, 2, 1),
-    GroupedVariant{256, 256, 512, rf::TileGeom<256, 256, 2, 4>::LDS_BYTES, rf::gemm_fp8_blockscale_grouped_mixed, true}};
+    RF_GROUPED(256, 256, 2, 4, 2), RF_GROUPED(128, 256, 2, 4, 3), RF_GROUPED(128, 128, 2, 2, 2), RF_GROUPED(128, 64, 2, 1, 2),
+    GroupedVariant{256, 256, 512, kMixedLds, rf::gemm_fp8_blockscale_grouped_mixed, true}};
 constexpr int kGroupedMixed = 4;
 constexpr int kNumGroupedVariants = sizeof(kGroupedVariants) / sizeof(kGroupedVariants[0]);
 

@@ -132,11 +132,15 @@ def main():
                     help="rewrite csrc/tuned_plans.inc, or PATH if given (rebuild libgemm.so afterwards)")
     ap.add_argument("--emit-file", default=None, help="append the best plan of every tuned shape to this plan file")
     ap.add_argument("--out", default=None)
+    ap.add_argument("--part", default=None, metavar="I/N", help="with --all: only every N-th shape, starting at the I-th (a sweep in N runs)")
     a = ap.parse_args()
     sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
     import radeonflow_kernels_amd as rfk
     rfk.lib()
     shapes = (SHAPES + (EXTENDED if a.extended else [])) if a.all else [(a.M, a.N, a.K)]
+    if a.part:
+        i, n_parts = (int(x) for x in a.part.split("/"))
+        shapes = shapes[i::n_parts]
     results = {}
     for (m, n, k) in shapes:
         cands = tune_shape(rfk, m, n, k)
