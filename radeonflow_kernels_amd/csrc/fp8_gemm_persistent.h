@@ -148,8 +148,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
                          :: "v"(goff_sb), "s"(src), "s"(lds_dst_sb), "n"(stage * STAGE_S) : "memory", "scc");
         }
     };
-    // The wait before the barrier is always vmcnt(0). Waiting for "all but the newest n loads" is not safe with
-    // LDS-DMA loads: a later load that hits in L2 was seen to complete before an earlier one that missed.
+    // Two stages: the wait before the barrier is for every load this wave has issued (the three-stage form of
+    // tile_mainloop, which waits for all but the newest block's loads, has no persistent counterpart: a tile would
+    // have to start on any of three stages).
     auto wait_for_stage = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
 
     // ---- LDS -> MFMA operands (see tile_mainloop) ----
