@@ -260,6 +260,11 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
         for (int d = TN; d < NDMA; d++) issue_dma(d, 1, dsrc[d]);
     }
 
+    // store instructions per wave of an unmasked tile store (store_whole_tile_bf16: one m-tile per pass, whole rows)
+    constexpr int NST = TM * (16 / (64 / (WN * 2 / 16)));
+    static_assert(NST <= 48, "the count must fit the wait instruction's field with room for the loads");
+    bool stores_behind = false;          // the newest NST vector memory instructions of this wave are a tile's stores
+
     // one K block of the current tile; cur = the LDS stage it reads
     // first_c: the first K block of a tile, whose cursor-1 loads have been issued already (before the previous tile's
     // store, see below)
@@ -274,7 +279,13 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
         for (int t = 0; t < NMFMA; t++) {
             const int j = t / TN, i = t % TN;
             if (t == BAR_SLOT) {
-                wait_for_stage();
+                // The first K block of a tile that follows a stored tile: the loads it waits for were all issued
+                // before that tile's stores, a wave's vector memory instructions complete in the order it issued
+                // them (loads and stores alike), so "all but the newest NST" are exactly the loads. The stores'
+                // acknowledgements (written through: about a microsecond under load) then have until the next K
+                // block's wait.
+                if (first && stores_behind) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NST) : "memory");
+                else wait_for_stage();
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -332,11 +343,14 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
         // the next tile (with two K blocks per tile: 0.7 us of each tile's 4.4).
 #pragma unroll
         for (int d = TN; d < NDMA; d++) issue_dma(d, 1, dsrc[d]);
-        if (m0_cur + BM <= M_store)
+        if (m0_cur + BM <= M_store) {
             store_whole_tile_bf16<BM, BN, WAVES_M, WAVES_N>(acc, C, N, m0_cur, n0_cur, lds + P::STAGING_OFF);
-        else                                              // the last rows of A are padding: C does not have them
+            stores_behind = true;
+        } else {                                          // the last rows of A are padding: C does not have them
             store_whole_tile_bf16<BM, BN, WAVES_M, WAVES_N, true>(acc, C, N, m0_cur, n0_cur, lds + P::STAGING_OFF,
                                                                   M_store - m0_cur);
+            stores_behind = false;                        // masked stores: how many were issued is not known here
+        }
 #pragma unroll
         for (int j = 0; j < TM; j++)
 #pragma unroll

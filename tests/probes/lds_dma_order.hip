@@ -1,9 +1,11 @@
-// Test infrastructure: do the LDS-DMA loads (global_load_lds_dwordx4) of one wave complete in issue order? Each
-// iteration a wave issues NA loads from a 1 GiB buffer (L2 misses: the addresses change every iteration) and then NB
-// loads from a small hot buffer (L2 hits), waits with s_waitcnt vmcnt(NB) and checks that the NA older loads have landed
-// in LDS (the buffer's content is a function of the address). A kernel that keeps more than one K block of loads in
-// flight and waits for "all but the newest n" relies on this. Prints one line per case; the last field of each line is
-// the number of stale dwords (expected 0).
+// Test infrastructure: do the vector memory instructions of one wave complete in issue order? Each iteration a wave
+// issues NA LDS-DMA loads (global_load_lds_dwordx4) from a 1 GiB buffer (L2 misses: the addresses change every
+// iteration) and then NB younger instructions that finish sooner: loads from a small hot buffer (L2 hits, 16 or 4 bytes
+// per lane), or stores of 16 bytes per lane to hot lines (plain, or written through with sc1). It waits with
+// s_waitcnt vmcnt(NB) and checks that the NA older loads have landed in LDS (the buffer's content is a function of the
+// address). The GEMM kernels rely on this twice: the three-stage loop waits for "all but the newest K block's loads",
+// and the persistent kernel's first wait of a tile for "all but the previous tile's stores". Prints one line per case;
+// the last field of each line is the number of stale dwords (expected 0).
 #include <hip/hip_runtime.h>
 #include <cstdio>
 #include <cstdlib>
@@ -36,7 +38,13 @@ __global__ __launch_bounds__(512) void probe(const uint32_t *big, size_t big_dwo
         }
 #pragma unroll
         for (int q = 0; q < NB; q++) {
-            if (WIDE_B)
+            if (WIDE_B == 2 || WIDE_B == 3) {
+                typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+                const u32x4_t w = {1u, 2u, 3u, (unsigned)it};
+                uint32_t *dst = (uint32_t *)hot + 4096 + ((blockIdx.x * 8 + wave) % 64) * 2048 + q * 256 + lane * 4;
+                if (WIDE_B == 2) asm volatile("global_store_dwordx4 %0, %1, off\n\ts_nop 1" :: "v"(dst), "v"(w) : "memory");
+                else asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" :: "v"(dst), "v"(w) : "memory");
+            } else if (WIDE_B)
                 asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" :: "v"(lane16), "s"(hot + q * 256), "s"(my + (NA + q) * 1024) : "memory");
             else
                 asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" :: "v"(lane4), "s"(hot + q * 256), "s"(my + (NA + q) * 1024) : "memory");
@@ -46,6 +54,8 @@ __global__ __launch_bounds__(512) void probe(const uint32_t *big, size_t big_dwo
         else if (NB == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
         else if (NB == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
         else if (NB == 7) asm volatile("s_waitcnt vmcnt(7)" ::: "memory");
+        else if (NB == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+        else if (NB == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
 #pragma unroll
         for (int q = 0; q < NA; q++) {
             volatile uint32_t *vp = (volatile uint32_t *)(lds + wave * (NA + NB) * 1024 + q * 1024 + lane * 16);
@@ -71,14 +81,14 @@ void run(const uint32_t *big, size_t n, const uint32_t *hot, int iters, unsigned
     float ms; CK(hipEventElapsedTime(&ms, e0, e1));
     printf("[%.1f ms, %.2f TB/s of misses] ", ms, 1024.0 * 8 * iters * NA * 1024 / (ms * 1e-3) / 1e12);
     unsigned long long h[2]; CK(hipMemcpy(h, d, 16, hipMemcpyDeviceToHost));
-    printf("older %d dwordx4 loads (L2 misses), then %d %s loads (L2 hits), wait vmcnt(%d): checked %llu stale %llu\n", NA, NB, WIDE_B ? "dwordx4" : "dword", NB, h[1], h[0]);
+    printf("older %d dwordx4 loads (L2 misses), then %d %s, wait vmcnt(%d): checked %llu stale %llu\n", NA, NB, WIDE_B == 2 ? "dwordx4 stores (L2 hits)" : WIDE_B == 3 ? "dwordx4 stores written through (sc1)" : WIDE_B ? "dwordx4 loads (L2 hits)" : "dword loads (L2 hits)", NB, h[1], h[0]);
     fflush(stdout);
 }
 int main(int argc, char **argv) {
     const int iters = argc > 1 ? atoi(argv[1]) : 2000;
     const size_t n = (size_t)1 << 28;   // 1 GiB of dwords: far larger than L2 + MALL
     uint32_t *big, *hot; unsigned long long *d;
-    CK(hipMalloc(&big, n * 4)); CK(hipMalloc(&hot, 16 * 1024)); CK(hipMalloc(&d, 16));
+    CK(hipMalloc(&big, n * 4)); CK(hipMalloc(&hot, 16 * 1024 + 64 * 2048 * 4 + 4096 * 4)); CK(hipMalloc(&d, 16));
     { std::vector<uint32_t> h(1 << 20); for (size_t c = 0; c < n; c += h.size()) { for (size_t i = 0; i < h.size(); i++) h[i] = pat(c + i); CK(hipMemcpy(big + c, h.data(), h.size() * 4, hipMemcpyHostToDevice)); } }
     CK(hipMemset(hot, 0x11, 16 * 1024));
     run<4, 0, 1>(big, n, hot, iters, d);     // control: vmcnt(0)
@@ -87,5 +97,10 @@ int main(int argc, char **argv) {
     run<4, 1, 1>(big, n, hot, iters, d);
     run<4, 1, 0>(big, n, hot, iters, d);     // the mixed-width case
     run<4, 4, 0>(big, n, hot, iters, d);
+    run<4, 4, 2>(big, n, hot, iters, d);     // younger stores that hit in L2
+    run<4, 16, 2>(big, n, hot, iters, d);
+    run<7, 8, 2>(big, n, hot, iters, d);
+    run<4, 16, 3>(big, n, hot, iters, d);    // younger stores written through to memory
+    run<7, 8, 3>(big, n, hot, iters, d);
     return 0;
 }

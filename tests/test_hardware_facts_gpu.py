@@ -86,16 +86,17 @@ def test_outputs_outside_the_reference_atol_are_explained_by_the_matrix_unit(nam
 
 def test_lds_dma_loads_of_a_wave_complete_in_issue_order():
     """global_load_lds_dwordx4 loads that miss L2 (random 1 KiB pieces of a 1 GiB buffer), followed by loads that hit
-    (16-byte and 4-byte ones), then s_waitcnt vmcnt(n) with n = the number of younger loads: the older loads' data is
-    in LDS every time. (The GEMM kernels wait with vmcnt(0) only; this keeps the fact on record for pipelines with
-    more than one K block of loads in flight.)"""
+    (16-byte and 4-byte ones) or stores that hit in L2 or are written through, then s_waitcnt vmcnt(n) with n = the
+    number of younger instructions: the older loads' data is in LDS every time. The three-stage loop (wait for all but
+    the newest K block's loads) and the persistent kernel's first wait of a tile (all but the previous tile's stores)
+    rely on it."""
     probe = os.path.join(HERE, "probes", "lds_dma_order")
     assert os.path.exists(probe), "build it with python tests/probes/build.py"
     p = subprocess.run([probe, "500"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=200)
     assert p.returncode == 0, p.stdout + p.stderr
     lines = [l for l in p.stdout.splitlines() if " stale " in l]
     print(p.stdout)
-    assert len(lines) == 6
+    assert len(lines) == 11
     for l in lines:
         f = l.split()
         assert int(f[f.index("checked") + 1]) > 10 ** 9 and int(f[f.index("stale") + 1]) == 0, l
