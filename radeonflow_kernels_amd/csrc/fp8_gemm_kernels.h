@@ -595,6 +595,12 @@ __device__ __forceinline__ void store_tile_bf16(const f32x4 (&acc)[BM / WAVES_M 
 // The staging region is written 8 bytes and read 16 bytes at a time: both through types that may alias anything, so
 // that the compiler keeps the writes (to its type rules an 8-byte vector store is never read by a 16-byte vector
 // load) and keeps them in order with the reads.
+// Store instructions a wave issues for one unmasked tile (one m-tile per pass, 64 / LPR rows per instruction).
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+constexpr int whole_tile_store_instructions() {
+    using G = TileGeom<BM, BN, WAVES_M, WAVES_N>;
+    return G::TM * (16 / (64 / (G::WN * 2 / 16)));
+}
 typedef uint32_t staged_u32x2 __attribute__((ext_vector_type(2), may_alias));
 typedef uint32_t staged_u32x4 __attribute__((ext_vector_type(4), may_alias));
 // MASKED: only the tile's first row_lim rows exist in C (a caller whose M is not a multiple of 16 has padded A and
@@ -608,6 +614,7 @@ __device__ __forceinline__ void store_whole_tile_bf16(const f32x4 (&acc)[BM / WA
     constexpr int LPR = G::WN * 2 / 16;                  // lanes per row on the way out (16 bytes each)
     static_assert(64 % LPR == 0 && 16 % (64 / LPR) == 0, "a store instruction covers whole rows of one m-tile");
     constexpr int RPI = 64 / LPR, NI = 16 / RPI;         // rows per store instruction, instructions per m-tile
+    static_assert(G::TM * NI == whole_tile_store_instructions<BM, BN, WAVES_M, WAVES_N>(), "the persistent kernel counts on it");
     int vz;                                              // see store_tile_bf16
     asm volatile("v_mov_b32 %0, 0" : "=v"(vz));
     const int lane = (threadIdx.x & 63) + vz, wave = threadIdx.x >> 6, L = lane & 15, g = lane >> 4;

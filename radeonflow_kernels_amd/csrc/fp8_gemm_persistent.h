@@ -261,7 +261,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
     }
 
     // store instructions per wave of an unmasked tile store (store_whole_tile_bf16: one m-tile per pass, whole rows)
-    constexpr int NST = TM * (16 / (64 / (WN * 2 / 16)));
+    constexpr int NST = whole_tile_store_instructions<BM, BN, WAVES_M, WAVES_N>();
     static_assert(NST <= 48, "the count must fit the wait instruction's field with room for the loads");
     bool stores_behind = false;          // the newest NST vector memory instructions of this wave are a tile's stores
 
