@@ -287,6 +287,35 @@ def test_benchmark_configs_full_size_sampled_rows_and_properties(rfk, name):
     assert torch.count_nonzero(g4[4]) == 0
 
 
+# the reference's benchmark shapes and seeds (scripts/problems/gemm/task.yml:66-84), its input style (bf16 normals cast
+# to fp8, signed normal scales)
+REFERENCE_BENCHMARKS = [(1024, 1536, 7168, 8135), (1024, 3072, 1536, 6251), (1024, 576, 7168, 12346),
+                        (1024, 7168, 256, 5364), (1024, 7168, 2048, 6132), (1024, 4608, 7168, 7531),
+                        (1024, 7168, 2304, 12345), (1024, 512, 7168, 6563), (1024, 4096, 512, 17512),
+                        (6144, 1536, 7168, 6543), (6144, 3072, 1536, 234), (6144, 576, 7168, 9863),
+                        (6144, 7168, 256, 764243), (6144, 7168, 2048, 76547), (6144, 4608, 7168, 65436),
+                        (6144, 7168, 2304, 452345), (6144, 512, 7168, 12341), (6144, 4096, 512, 45245)]
+
+
+@pytest.mark.parametrize("m,n,k,seed", REFERENCE_BENCHMARKS)
+def test_reference_benchmark_shapes_sampled_rows(rfk, m, n, k, seed):
+    """Every benchmark shape of the reference under its tabled plan: 48 sampled rows (tile edges among them) against
+    the oracle at the graded tolerance, few mismatches at the reference harness's atol, canary intact."""
+    data = rk.generate_input_reference_style(m, n, k, seed)
+    g, buf = to_gpu(data, canary_elems=1024)
+    rfk.fp8_mm(*g)
+    torch.cuda.synchronize()
+    assert np.all(buf[g[4].numel():].float().cpu().numpy() == -7.0), "store past the end of C"
+    rng = np.random.default_rng(seed)
+    rows = np.unique(np.concatenate([[0, 1, 127, 128, 255, 256, m - 1], rng.integers(0, m, 41)])).astype(np.int32)
+    a, b, sa, sb = rk.raw_layouts(data)
+    _, exp16 = cref.ref_gemm_f32(a, b, sa, sb, rows=rows)
+    got = g[4][torch.from_numpy(rows).long().cuda()]
+    what = "%dx%dx%d" % (m, n, k)
+    assert_close_to_oracle(got, exp16, RTOL, ATOL, what)
+    assert_few_mismatches_at_reference_atol(got, exp16, what)
+
+
 def test_run_entry_writes_metrics_from_the_stream_callback(rfk):
     from radeonflow_kernels_amd import gemm
     data = rk.generate_input_blockquant(256, 256, 512, 3)
