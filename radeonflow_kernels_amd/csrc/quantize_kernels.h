@@ -304,18 +304,24 @@ __device__ __forceinline__ void quantize_block128_body(const void *__restrict__ 
     for (int g = 0; g < NG; g++)
 #pragma unroll
         for (int e = 0; e < KPT; e++) {
-            float yu[4], yd[4];
+            // bf16 sources go straight to the exact quotient: x and amax have 8-bit mantissas, so x / scale often IS
+            // a rounding boundary, one such lane in 64 sends the whole wave to the exact path, and with 256 values per
+            // wave and group that is nearly every time; the bracket would only be computed on top of it.
+            int hi = 0, lo = 1;
+            if constexpr (!IN_BF16) {
+                float yu[4], yd[4];
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                yu[j] = v[4 * g + j][e] * rup[4 * g + j];
-                yd[j] = v[4 * g + j][e] * rdown[4 * g + j];
+                for (int j = 0; j < 4; j++) {
+                    yu[j] = v[4 * g + j][e] * rup[4 * g + j];
+                    yd[j] = v[4 * g + j][e] * rdown[4 * g + j];
+                }
+                // (the first conversion of a word keeps the upper half of its old value, which the second one
+                // overwrites: any register will do as the old value)
+                hi = __builtin_amdgcn_cvt_pk_fp8_f32(yu[0], yu[1], __builtin_bit_cast(int, yu[0]), false);
+                hi = __builtin_amdgcn_cvt_pk_fp8_f32(yu[2], yu[3], hi, true);
+                lo = __builtin_amdgcn_cvt_pk_fp8_f32(yd[0], yd[1], __builtin_bit_cast(int, yd[0]), false);
+                lo = __builtin_amdgcn_cvt_pk_fp8_f32(yd[2], yd[3], lo, true);
             }
-            // (the first conversion of a word keeps the upper half of its old value, which the second one overwrites:
-            // any register will do as the old value)
-            int hi = __builtin_amdgcn_cvt_pk_fp8_f32(yu[0], yu[1], __builtin_bit_cast(int, yu[0]), false);
-            hi = __builtin_amdgcn_cvt_pk_fp8_f32(yu[2], yu[3], hi, true);
-            int lo = __builtin_amdgcn_cvt_pk_fp8_f32(yd[0], yd[1], __builtin_bit_cast(int, yd[0]), false);
-            lo = __builtin_amdgcn_cvt_pk_fp8_f32(yd[2], yd[3], lo, true);
             uint32_t w = (uint32_t)hi;
             if (__builtin_expect(!fast[g], 0)) {
                 w = f32x4_to_e4m3fn_codes(v[4 * g][e] / s[4 * g], v[4 * g + 1][e] / s[4 * g + 1],
