@@ -5,6 +5,8 @@
 // variant table tuned for gfx950) instead of a switch over 29 hard-coded shapes, and no transpose
 // pre-pass or transposed copies exist.
 #include <hip/hip_runtime.h>
+#include <algorithm>
+#include <cmath>
 
 #include <cstdio>
 #include <cstdlib>
@@ -1054,19 +1056,36 @@ int grouped_gemm(const void *a, const void *b, const float *as, const float *bs,
             if (t > most) { most = t; most_v = v; }
         }
         if (variant < 0) variant = most_v;
-        // Every row tile of a group streams the group's whole weight block, and with small groups that traffic is the
-        // bound. 128-row tiles are the better choice exactly when they do not add row tiles (nearly all groups have at
-        // most 128 rows): same weight traffic, half the padding. Measured, N=4096 K=7168: 32 groups of 16..128 rows
-        // 186-202 us against 219-233 us; 64 groups of 16..176 rows (a third of them above 128) 505 against 457 us.
+        // Enough tiles for the 256-wide family: 256-row tiles, 128-row tiles (three stages) or the mixed form, by a
+        // small model of what was measured (N = 4096, K = 7168, twelve group layouts). A tile costs its compute
+        // (91 for 256 rows, 52 for 128, arbitrary units) plus a share of streaming its column tile of the group's
+        // weights (36, divided among the row tiles that use it: they run side by side on one XCD); the launch takes
+        // as many rounds of one tile per CU as the tile count needs, a last partial round counting 0.6 + 0.4 x its
+        // fill. Round counts decide most cases: 32 uneven groups of 16..816 rows are 816 mixed tiles (3.19 rounds,
+        // 369 us) or 1280 tiles of 128 rows (5.00 rounds, 342 us); 20 groups of 384 rows 287 against 246 us; 64 groups
+        // of 16..176 rows 408 against 447 us. On the twelve layouts the choice is 0.9 % slower than the best of the
+        // three on average, 8 % at worst (always taking the mixed form: 2.6 % and 17 %).
         if (variant == 0) {
-            long t256 = 0, t128 = 0;
-            for (int g = 0; g < groups; g++) {
-                const int rows = row_offsets[g + 1] - row_offsets[g];
-                t256 += ceil_div(rows, 256);
-                t128 += ceil_div(rows, 128);
+            const int tiles_n256 = ceil_div(n, 256);
+            double best_t = 0;
+            for (int cand : {0, 1, kGroupedMixed}) {
+                double cost = 0;
+                long items = 0;
+                for (int g = 0; g < groups; g++) {
+                    const int rows = row_offsets[g + 1] - row_offsets[g];
+                    if (rows == 0) continue;
+                    int big, small;
+                    if (cand == 0) { big = ceil_div(rows, 256); small = 0; }
+                    else if (cand == 1) { big = 0; small = ceil_div(rows, 128); }
+                    else { big = rows / 256 + (rows % 256 > 128 ? 1 : 0); small = rows % 256 > 0 && rows % 256 <= 128 ? 1 : 0; }
+                    cost += tiles_n256 * (91.0 * big + 52.0 * small + 36.0);      // 36 / t for each of the t row tiles
+                    items += (long)tiles_n256 * (big + small);
+                }
+                const double rounds_exact = (double)items / s.num_cu;
+                const double full = std::floor(rounds_exact), frac = rounds_exact - full;
+                const double t = (full + (frac > 0 ? 0.6 + 0.4 * frac : 0.0)) * cost / (double)items;
+                if (best_t == 0 || t < best_t) { best_t = t; variant = cand; }
             }
-            if (t128 * 20 <= t256 * 21 && t128 * ceil_div(n, 256) >= s.num_cu) variant = 1;
-            else variant = kGroupedMixed;      // same tiles as 256x256, but a short left-over costs half
         }
     }
     const GroupedVariant &v = kGroupedVariants[variant];
