@@ -1056,7 +1056,9 @@ int grouped_gemm(const void *a, const void *b, const float *as, const float *bs,
             if (t > most) { most = t; most_v = v; }
         }
         if (variant < 0) variant = most_v;
-        // Enough tiles for the 256-wide family: 256-row tiles, 128-row tiles (three stages) or the mixed form, by a
+        if (variant == 1) variant = 0;      // 128-row tiles fill the chip: the 256-wide family, chosen below
+        // Enough tiles for the 256-wide family (128-row tiles would give every CU one): 256-row tiles, 128-row tiles
+        // (three stages) or the mixed form, by a
         // small model of what was measured (N = 4096, K = 7168, twelve group layouts). A tile costs its compute
         // (91 for 256 rows, 52 for 128, arbitrary units) plus a share of streaming its column tile of the group's
         // weights (36, divided among the row tiles that use it: they run side by side on one XCD); the launch takes
