@@ -45,7 +45,7 @@ enum {
     RF_ERR_BAD_CONFIG = 4      /* explicit config not available for this shape */
 };
 
-enum { RF_SCHEDULE_TILES = 0, RF_SCHEDULE_STREAM_K = 1, RF_SCHEDULE_PERSISTENT = 2 };
+enum { RF_SCHEDULE_TILES = 0, RF_SCHEDULE_STREAM_K = 1, RF_SCHEDULE_PERSISTENT = 2, RF_SCHEDULE_PERSISTENT_HALF_TAIL = 3 };
 
 /* One launch plan: which kernel variant and how K is split.
  * Replaces a DISPATCH_GEMM(...) line of the reference (src/gemm/gemm_launcher.cpp:158-162,229-259). */
@@ -59,7 +59,11 @@ typedef struct rf_gemm_config {
                                       line; needs split_k == 1 and at least as many tiles as CUs;
                          2 PERSISTENT persistent grid, whole tiles, one load/compute pipeline running across the
                                       tiles of a workgroup; needs split_k == 1, M a multiple of 16 and at least the
-                                      tile height, N a multiple of the tile width, K/128 even */
+                                      tile height, N a multiple of the tile width, K/128 even;
+                         3 PERSISTENT_HALF_TAIL  the persistent schedule for the whole rounds of one tile per CU, the
+                                      left-over tiles finished as 128-row half tiles, one per CU; 256x256 tile only,
+                                      needs the persistent schedule's shape rules, at least one tile per CU and a
+                                      last round that is at most half full */
 } rf_gemm_config;
 
 /* Drop-in for the reference's launcher entry (src/gemm/gemm_launcher.cpp:182-184):

@@ -30,7 +30,13 @@ struct PersistentGeom {
     static_assert(LDS_BYTES <= 160 * 1024, "stages + private store regions fit the CU's LDS");
 };
 
-template <int BM, int BN, int WAVES_M, int WAVES_N>
+// HALF_TAIL (256 x 256 tiles): the grid's workgroups take the whole rounds only (the first T - T % grid tiles), and the
+// T % grid tiles that are left are finished as 128 x 256 half tiles, one per workgroup, by the three-stage loop of
+// tile_mainloop: a last round that is at most half full then takes about half a tile's time instead of a whole one
+// (8192 x 4608 x 7168 is 576 tiles on 256 CUs: 2.25 rounds). Left-over tile i (0 <= i < R) is split between workgroups
+// i and i + R8, R8 = R rounded up to a multiple of 8, so that both run on the XCD whose region the tile belongs to;
+// the host checks 0 < R and R8 + R <= grid.
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool HALF_TAIL = false>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_persistent(
     const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
     const float *__restrict__ SB, uint16_t *__restrict__ C, int M, int N, int K, int tiles_m, int tiles_n,
@@ -56,7 +62,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
     const int wm = wave % WAVES_M, wn = wave / WAVES_M;
     const int QK = K / BK, QN = (N + 127) / 128;
     const int T = tiles_m * tiles_n;
-    const int my_tiles =                                                                // >= 1: grid <= T
+    const int my_tiles = HALF_TAIL ? T / (int)gridDim.x :                               // >= 1: grid <= T
         __builtin_amdgcn_readfirstlane((T - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x);
 
     // Origin of this workgroup's r-th tile; past the end it repeats the last one (prefetches that nobody uses). The map
@@ -364,6 +370,22 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
     }
     // prefetches past the last tile must land before the LDS is handed on
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if constexpr (HALF_TAIL) {
+        static_assert(BM == 256 && BN == 256 && WAVES_M == 2 && WAVES_N == 4, "half tiles of the 256 x 256 tile");
+        const int grid = (int)gridDim.x, R = T % grid, R8 = (R + 7) / 8 * 8;
+        const int b = (int)blockIdx.x;
+        const int half = b < R ? 0 : (b >= R8 && b < R8 + R) ? 1 : -1;
+        if (half < 0) return;                               // uniform over the workgroup
+        int tm, tn;
+        tile_of_block(T - R + (half ? b - R8 : b), T, tiles_m, tiles_n, group_m, true, tm, tn);
+        const int m0 = (tm * BM < M - BM ? tm * BM : M - BM) + 128 * half, n0 = tn * BN;
+        __syncthreads();                                    // every wave is done with its store staging region
+        using H = TileGeom<128, 256, 2, 4, 3>;
+        static_assert(H::LDS_BYTES <= P::LDS_BYTES, "the half tile's stages fit this kernel's LDS");
+        f32x4 acc2[H::TM][H::TN];
+        tile_mainloop<128, 256, 2, 4, 3>(A, B, SA, SB, M, M, N, m0, n0, 0, QK, lds, acc2);
+        store_tile_bf16<128, 256, 2, 4>(acc2, C, M_store, N, m0, n0, lds);
+    }
 }
 
 }  // namespace rf

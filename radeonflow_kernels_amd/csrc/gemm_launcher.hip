@@ -54,6 +54,7 @@ struct Variant {
     streamk_kernel_t streamk;            // null: the variant has no stream-K form
     persistent_kernel_t persistent;      // null: no persistent form
     int lds_persistent;
+    persistent_kernel_t persistent_half_tail = nullptr;   // null: no form that ends with half tiles
     int lds_bytes() const { return lds; }
     int threads() const { return waves_m * waves_n * 64; }
 };
@@ -79,7 +80,10 @@ struct Variant {
               rf::gemm_fp8_blockscale_tile<BM, BN, WM, WN, false, 3>,                      \
               rf::gemm_fp8_blockscale_tile<BM, BN, WM, WN, true, 3>, nullptr, nullptr, 0 }
 const Variant kVariants[] = {
-    RF_VARIANT(256, 256, 2, 4),   // 0: 8 waves, wave tile 128(m) x 64(n), 128 KiB LDS
+    Variant{256, 256, 2, 4, rf::TileGeom<256, 256, 2, 4>::LDS_BYTES, rf::gemm_fp8_blockscale_tile<256, 256, 2, 4, false>,
+            rf::gemm_fp8_blockscale_tile<256, 256, 2, 4, true>, rf::gemm_fp8_blockscale_streamk<256, 256, 2, 4>,
+            rf::gemm_fp8_blockscale_persistent<256, 256, 2, 4>, rf::PersistentGeom<256, 256, 2, 4>::LDS_BYTES,
+            rf::gemm_fp8_blockscale_persistent<256, 256, 2, 4, true>},   // 0: 8 waves, wave tile 128(m) x 64(n), 128 KiB LDS
     RF_VARIANT(128, 128, 2, 2),   // 1: 4 waves, wave tile 64 x 64, 64 KiB LDS (2 workgroups per CU)
     RF_VARIANT(256, 128, 2, 2),   // 2: 4 waves, wave tile 128 x 64, 96 KiB LDS
     RF_VARIANT(128, 256, 2, 4),   // 3: 8 waves, wave tile 64 x 64, 96 KiB LDS
@@ -166,7 +170,7 @@ int parse_plans(const char *path, std::vector<TunedPlan> &out) {
         if (got <= 0) continue;                       // blank or comment line
         if (got != 7 || p.m < 1 || p.n < 1 || p.k < rf::BK || p.k % rf::BK != 0 || p.variant < 0 ||
             p.variant >= kNumVariants || p.split_k < 1 || p.group_m < 1 || p.stream_k < RF_SCHEDULE_TILES ||
-            p.stream_k > RF_SCHEDULE_PERSISTENT || (p.stream_k != RF_SCHEDULE_TILES && p.split_k != 1)) {
+            p.stream_k > RF_SCHEDULE_PERSISTENT_HALF_TAIL || (p.stream_k != RF_SCHEDULE_TILES && p.split_k != 1)) {
             fclose(f);
             return fail(RF_ERR_BAD_CONFIG, std::string(path) + ":" + std::to_string(lineno) +
                                                ": expected \"M N K variant split_k group_m stream_k\" with valid values");
@@ -202,6 +206,9 @@ int ensure_device_info(State &s) {
             RF_HIP(hipFuncSetAttribute((const void *)v.streamk, hipFuncAttributeMaxDynamicSharedMemorySize, v.lds_bytes()));
         if (v.persistent)
             RF_HIP(hipFuncSetAttribute((const void *)v.persistent, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       v.lds_persistent));
+        if (v.persistent_half_tail)
+            RF_HIP(hipFuncSetAttribute((const void *)v.persistent_half_tail, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        v.lds_persistent));
     }
     // the device address of this device's copy of the scratch array (the array's name is only a host-side handle)
@@ -334,6 +341,15 @@ bool persistent_ok(const Variant &v, int m, int n, int k) {
     return v.persistent && m >= v.bm && m % 16 == 0 && n % v.bn == 0 && (k / rf::BK) % 2 == 0;
 }
 
+// Persistent schedule that finishes the last, partial round with half tiles: one workgroup per CU, at least one whole
+// round, and a last round that two half tiles per left-over tile still fit into (see the kernel).
+bool half_tail_ok(const Variant &v, int m, int n, int k, int num_cu) {
+    if (!v.persistent_half_tail || !persistent_ok(v, m, n, k)) return false;
+    const long t = (long)ceil_div(m, v.bm) * ceil_div(n, v.bn);
+    const long r = t % num_cu;
+    return t >= num_cu && r > 0 && (r + 7) / 8 * 8 + r <= num_cu;
+}
+
 // Stream-K: at least one tile per workgroup (then a split tile has exactly two contributors, which is all the kernel
 // handles) and no more tiles than arrival counters.
 bool stream_k_ok(const Variant &v, int m, int n, int num_cu) {
@@ -362,7 +378,8 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
     auto usable = [&](const TunedPlan &p) {
         return p.m == m && p.n == n && p.k == k && p.variant < kNumVariants && p.split_k <= k / rf::BK &&
                (p.stream_k != RF_SCHEDULE_PERSISTENT || persistent_ok(kVariants[p.variant], m, n, k)) &&
-               (p.stream_k != RF_SCHEDULE_STREAM_K || stream_k_ok(kVariants[p.variant], m, n, num_cu));
+               (p.stream_k != RF_SCHEDULE_STREAM_K || stream_k_ok(kVariants[p.variant], m, n, num_cu)) &&
+               (p.stream_k != RF_SCHEDULE_PERSISTENT_HALF_TAIL || half_tail_ok(kVariants[p.variant], m, n, k, num_cu));
     };
     const TunedPlan *hit = nullptr;
     for (const TunedPlan &p : user_plans)
@@ -380,6 +397,8 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
     // 103 shapes its plan is 0.8 % slower than the best measured one on average, 8 % at worst). Time in microseconds of a plan =
     //   rounds * (K blocks per workgroup * c + f)           one workgroup per tile and K split
     //   rounds * K blocks * c + f + (rounds - 1) * f_next   persistent: only the first tile starts cold
+    //   the same over the whole rounds + f_next + K blocks * c of the three-stage 128x256 tile
+    //                                                       persistent with a last round of half tiles
     //   + reduction cost when K is split
     // with rounds = ceil(workgroups / CUs). Candidates: the 256x256 tile and the 128x256, 192x192, 128x192 and 64x128
     // tiles with two and with three stages (192-wide tiles win where they divide the shape into fuller rounds or leave
@@ -388,7 +407,7 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
     struct Candidate { int variant; double c, f; };
     const Candidate cands[] = {{0, 0.955, 7.96}, {3, 0.619, 5.11}, {5, 0.71, 5.2},  {6, 0.74, 3.7},  {7, 0.82, 0.0},
                                {8, 0.52, 4.5},   {9, 0.70, 0.5},   {10, 0.53, 5.9}, {11, 0.62, 5.8}};
-    const double f_next = 3.0, reduce_fixed = 2.83, reduce_per_elem = 1.37e-6;
+    const double f_next = 3.0, reduce_fixed = 2.83, reduce_per_elem = 1.37e-6, c_half_tile = 0.53;
     const int splits_tried[] = {1, 2, 3, 4, 6, 8, 12, 16};
     const int qk = k / rf::BK;
     double best_cost = 1e30;
@@ -409,6 +428,15 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
                     out->variant = cd.variant;
                     out->split_k = sp;
                     out->stream_k = sched;
+                }
+                if (sched == RF_SCHEDULE_PERSISTENT && half_tail_ok(v, m, n, k, num_cu)) {
+                    t = (rounds - 1) * kb_per * cd.c + cd.f + (rounds - 1) * f_next + kb_per * c_half_tile;
+                    if (t < best_cost) {
+                        best_cost = t;
+                        out->variant = cd.variant;
+                        out->split_k = 1;
+                        out->stream_k = RF_SCHEDULE_PERSISTENT_HALF_TAIL;
+                    }
                 }
             }
         }
@@ -437,6 +465,11 @@ int launch_locked(State &s, Mem &mem, const void *a, const void *b, const float 
         } else if (cfg.stream_k == RF_SCHEDULE_PERSISTENT) {
             if (!persistent_ok(kVariants[cfg.variant], m, n, k))
                 return fail(RF_ERR_BAD_CONFIG, "the persistent schedule needs M >= the tile height, M % 16 == 0, N a multiple of the tile width and K/128 even");
+        } else if (cfg.stream_k == RF_SCHEDULE_PERSISTENT_HALF_TAIL) {
+            if (!half_tail_ok(kVariants[cfg.variant], m, n, k, s.num_cu))
+                return fail(RF_ERR_BAD_CONFIG, "the half-tile schedule needs the 256x256 tile, the persistent schedule's "
+                                               "shape rules, at least one tile per compute unit and a last round that "
+                                               "is at most half full");
         } else if (cfg.stream_k != RF_SCHEDULE_TILES) {
             return fail(RF_ERR_BAD_CONFIG, "unknown schedule");
         }
@@ -471,6 +504,12 @@ int launch_locked(State &s, Mem &mem, const void *a, const void *b, const float 
         hipLaunchKernelGGL(v.persistent, dim3(T < P ? T : P), block, v.lds_persistent, stream,
                            (const uint8_t *)a, (const uint8_t *)b, as, bs, (uint16_t *)c, m, n, k, tiles_m, tiles_n,
                            cfg.group_m, m_store);
+        RF_HIP(hipGetLastError());
+        return RF_OK;
+    }
+    if (cfg.stream_k == RF_SCHEDULE_PERSISTENT_HALF_TAIL) {
+        hipLaunchKernelGGL(v.persistent_half_tail, dim3(s.num_cu), block, v.lds_persistent, stream, (const uint8_t *)a,
+                           (const uint8_t *)b, as, bs, (uint16_t *)c, m, n, k, tiles_m, tiles_n, cfg.group_m, m_store);
         RF_HIP(hipGetLastError());
         return RF_OK;
     }

@@ -77,12 +77,17 @@ def tune_shape(rfk, m, n, k, log=print):
     ncu = torch.cuda.get_device_properties(0).multi_processor_count
     for v in rfk.variants():
         tiles = -(-m // v["block_m"]) * -(-n // v["block_n"])
-        # schedules: 0 = one workgroup per tile (with K splits), 1 = stream-K, 2 = persistent whole tiles
-        for split, sk in [(sp, 0) for sp in SPLITS] + [(1, 1), (1, 2)]:
+        # schedules: 0 = one workgroup per tile (with K splits), 1 = stream-K, 2 = persistent whole tiles,
+        # 3 = persistent with a last round of half tiles
+        for split, sk in [(sp, 0) for sp in SPLITS] + [(1, 1), (1, 2), (1, 3)]:
             if split > k // 128 or (sk == 1 and (tiles < ncu or not v["stream_k"])):
                 continue
-            if sk == 2 and (not v["persistent"] or m < v["block_m"] or m % 16 or n % v["block_n"] or (k // 128) % 2):
+            if sk in (2, 3) and (not v["persistent"] or m < v["block_m"] or m % 16 or n % v["block_n"] or (k // 128) % 2):
                 continue
+            if sk == 3:
+                left = tiles % ncu
+                if v["variant"] != 0 or tiles < ncu or left == 0 or (left + 7) // 8 * 8 + left > ncu:
+                    continue
             for gm in GROUPS:
                 cfg = rfk.GemmConfig(v["variant"], split, gm, sk)
                 args[4].zero_()

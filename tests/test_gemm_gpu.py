@@ -202,6 +202,59 @@ def test_large_m_that_is_not_a_tile_multiple_runs_the_persistent_plan_automatica
     assert np.array_equal(bf16_bits(out), oracle_bf16(data))
 
 
+@pytest.mark.parametrize("m,n,k", [(4608, 4096, 256), (4352, 4096, 512), (4592, 4096, 256), (2320, 8192, 256),
+                                   (8192, 4608, 256)])
+def test_persistent_schedule_with_a_last_round_of_half_tiles(rfk, m, n, k):
+    """More tiles than CUs and a last round that is at most half full (32, 16, 32, 64 and 64 left-over tiles on 256
+    CUs; 4592 and 2320 rows also end on a tile row that overlaps the one before): the left-over tiles are computed as
+    upper and lower halves by two workgroups each. Exact data against the oracle, bit for bit, twice; then data with
+    rounding in it against the one-workgroup-per-tile kernel, bit for bit and the same on every launch."""
+    if torch.cuda.get_device_properties(0).multi_processor_count != 256:
+        pytest.skip("left-over counts are worked out for 256 compute units")
+    data = exact_problem(m, n, k, seed=m + 3 * n + k)
+    exp = oracle_bf16(data)
+    for gm in (1, 8):
+        cfg = rfk.GemmConfig(0, 1, gm, 3)
+        for rep in range(2):
+            out = _run(rfk, data, config=cfg, canary=1024)
+            assert np.array_equal(bf16_bits(out), exp), "plan %r rep %d" % (cfg, rep)
+    noisy = rk.generate_input_blockquant(m, n, k, seed=m + k)
+    tiles = bf16_bits(_run(rfk, noisy, config=rfk.GemmConfig(0, 1, 8, 0), canary=1024)).copy()
+    for rep in range(3):
+        out = _run(rfk, noisy, config=rfk.GemmConfig(0, 1, 8, 3), canary=1024)
+        assert np.array_equal(bf16_bits(out), tiles), "rep %d differs from the tile kernel" % rep
+
+
+def test_half_tile_schedule_under_a_ragged_m_writes_c_in_place(rfk, tmp_path):
+    """4593 rows: the operands are staged with 4608 rows and the plan of the padded shape, here the half-tile
+    schedule, stores only the true rows (the lower half tiles of the last tile row are masked by row)."""
+    m, n, k = 4593, 4096, 256
+    path = tmp_path / "p.plans"
+    path.write_text("4608 %d %d 0 1 8 3\n" % (n, k))
+    data = exact_problem(m, n, k, seed=78)
+    try:
+        assert rfk.load_plans(str(path)) == 1
+        got = rfk.select_config(4608, n, k)
+        if got.stream_k != 3:
+            pytest.skip("the half-tile schedule does not fit this device's CU count")
+        for rep in range(2):
+            out = _run(rfk, data, canary=8192)
+            assert np.array_equal(bf16_bits(out), oracle_bf16(data)), "rep %d" % rep
+    finally:
+        rfk.clear_plans()
+
+
+def test_half_tile_schedule_rejects_shapes_it_does_not_fit(rfk):
+    for m, n, k, variant in [(2048, 2048, 256, 0),      # fewer tiles than CUs
+                             (8192, 2048, 256, 0),      # 256 tiles: no last round
+                             (6144, 4608, 256, 0),      # 432 tiles: last round more than half full
+                             (4608, 4096, 384, 0),      # three K blocks
+                             (4608, 4096, 256, 3)]:     # not the 256 x 256 tile
+        data = exact_problem(m, n, k, seed=1)
+        with pytest.raises(RuntimeError):
+            _run(rfk, data, config=rfk.GemmConfig(variant, 1, 8, 3))
+
+
 def test_persistent_schedule_rejects_ragged_shapes(rfk):
     data = exact_problem(272, 144, 256, seed=1)
     with pytest.raises(RuntimeError):
