@@ -397,8 +397,10 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
     // 103 shapes its plan is 0.8 % slower than the best measured one on average, 8 % at worst). Time in microseconds of a plan =
     //   rounds * (K blocks per workgroup * c + f)           one workgroup per tile and K split
     //   rounds * K blocks * c + f + (rounds - 1) * f_next   persistent: only the first tile starts cold
-    //   the same over the whole rounds + f_next + K blocks * c of the three-stage 128x256 tile
-    //                                                       persistent with a last round of half tiles
+    //   the same over the whole rounds + f_next + K blocks * c + f of the three-stage 128x256 tile
+    //                                                       persistent with a last round of half tiles (the half
+    //                                                       tiles start cold: at K = 512 the plain persistent
+    //                                                       schedule of 128x256 tiles is 15-20 % faster)
     //   + reduction cost when K is split
     // with rounds = ceil(workgroups / CUs). Candidates: the 256x256 tile and the 128x256, 192x192, 128x192 and 64x128
     // tiles with two and with three stages (192-wide tiles win where they divide the shape into fuller rounds or leave
@@ -407,7 +409,7 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
     struct Candidate { int variant; double c, f; };
     const Candidate cands[] = {{0, 0.955, 7.96}, {3, 0.619, 5.11}, {5, 0.71, 5.2},  {6, 0.74, 3.7},  {7, 0.82, 0.0},
                                {8, 0.52, 4.5},   {9, 0.70, 0.5},   {10, 0.53, 5.9}, {11, 0.62, 5.8}};
-    const double f_next = 3.0, reduce_fixed = 2.83, reduce_per_elem = 1.37e-6, c_half_tile = 0.53;
+    const double f_next = 3.0, reduce_fixed = 2.83, reduce_per_elem = 1.37e-6, c_half_tile = 0.53, f_half_tile = 4.0;
     const int splits_tried[] = {1, 2, 3, 4, 6, 8, 12, 16};
     const int qk = k / rf::BK;
     double best_cost = 1e30;
@@ -430,7 +432,7 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
                     out->stream_k = sched;
                 }
                 if (sched == RF_SCHEDULE_PERSISTENT && half_tail_ok(v, m, n, k, num_cu)) {
-                    t = (rounds - 1) * kb_per * cd.c + cd.f + (rounds - 1) * f_next + kb_per * c_half_tile;
+                    t = (rounds - 1) * kb_per * cd.c + cd.f + (rounds - 1) * f_next + kb_per * c_half_tile + f_half_tile;
                     if (t < best_cost) {
                         best_cost = t;
                         out->variant = cd.variant;

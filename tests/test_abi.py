@@ -135,8 +135,8 @@ def test_plan_files_parse_without_a_device(tmp_path):
 
 def test_compiled_in_plan_table_only_holds_plans_its_shapes_can_run():
     """Every line of csrc/tuned_plans.inc names an existing variant, a split that leaves every part at least one K
-    block, and the persistent schedule only where the tile divides the shape and K/128 is even (a plan that cannot
-    run is skipped at lookup, so a bad line would silently fall back to the cost model)."""
+    block, and the persistent schedules only where the shape allows them (a plan that cannot run is skipped at lookup,
+    so a bad line would silently fall back to the cost model)."""
     from radeonflow_kernels_amd import gemm
     L = gemm.lib()
     inc = os.path.join(ROOT, "radeonflow_kernels_amd", "csrc", "tuned_plans.inc")
@@ -146,10 +146,16 @@ def test_compiled_in_plan_table_only_holds_plans_its_shapes_can_run():
         bm, bn = ctypes.c_int(), ctypes.c_int()
         assert L.rf_gemm_variant_info(variant, ctypes.byref(bm), ctypes.byref(bn), None, None, None) == 0
         assert m % 16 == 0 and n % 16 == 0 and k % 128 == 0 and 1 <= split <= k // 128 and group >= 1
-        assert schedule in (0, 2), "the stream-K schedule is never tabled"
-        if schedule == 2:
+        assert schedule in (0, 2, 3), "the stream-K schedule is never tabled"
+        if schedule in (2, 3):
             assert L.rf_gemm_variant_has_persistent(variant) == 1 and split == 1
-            assert m % bm.value == 0 and n % bn.value == 0 and (k // 128) % 2 == 0
+            assert m >= bm.value and n % bn.value == 0 and (k // 128) % 2 == 0
+        if schedule == 3:
+            # measured on 256 compute units: whole rounds first, then a last round that is at most half full (on a
+            # device with another count the plan is checked again at lookup and skipped if it does not fit)
+            tiles = -(-m // 256) * (n // 256)
+            left = tiles % 256
+            assert variant == 0 and tiles >= 256 and 0 < left and (left + 7) // 8 * 8 + left <= 256
 
 
 def test_tuner_never_writes_a_stream_k_winner_into_a_table_or_plan_file(tmp_path):
