@@ -41,6 +41,11 @@ CONFIGS = {
     "C4": (6144, 7168, 256, 764243),
     "C5": (1024, 576, 7168, 12346),
 }
+# measured only when named with --config (not part of the default run): a shape whose last round of 256x256 tiles is
+# a quarter full, the automatic plan of which is the persistent schedule with a last round of half tiles
+EXTRA_CONFIGS = {
+    "H1": (8192, 4608, 7168, 4321),
+}
 RTOL, ATOL, ATOL_REFERENCE = 2e-2, 1e-2, 1e-3
 SETTLE_SECONDS = 0.4
 KERNEL_SOURCES = ("fp8_gemm_kernels.h", "fp8_gemm_persistent.h")
@@ -231,7 +236,7 @@ def parity_report(rfk, cref, rk, data, g, stream, expect=None, truth_rows=64):
 def measure_config(rfk, cref, rk, name, steps, warmup, stream, with_cpu, settle_seconds, keep=False):
     """One configuration: inputs, settled launch time, roofline fraction, correctness gate. Returns the record (and
     the inputs with keep=True)."""
-    m, n, k, seed = CONFIGS[name]
+    m, n, k, seed = {**CONFIGS, **EXTRA_CONFIGS}[name]
     t0 = time.time()
     data = rk.generate_input_blockquant(m, n, k, seed)
     g = to_gpu(data)
@@ -239,7 +244,8 @@ def measure_config(rfk, cref, rk, name, steps, warmup, stream, with_cpu, settle_
     cold = rfk.fp8_mm_time(*g, warmup=warmup, iters=steps) if keep else None     # the process's first launches
     us, settle = settled_us(rfk, g, steps, warmup, settle_seconds)
     cfg = rfk.select_config(m, n, k)
-    schedule = {0: "gemm_fp8_blockscale_tile", 1: "gemm_fp8_blockscale_streamk", 2: "gemm_fp8_blockscale_persistent"}
+    schedule = {0: "gemm_fp8_blockscale_tile", 1: "gemm_fp8_blockscale_streamk", 2: "gemm_fp8_blockscale_persistent",
+                3: "gemm_fp8_blockscale_persistent with a last round of half tiles"}
     launches = 1 if cfg.split_k == 1 else 2
     rec = {"shape": [m, n, k], "us_per_gemm": round(us, 2), "settle_launches": settle,
            "tflops": round(2.0 * m * n * k / us / 1e6, 1), "gbs_algorithmic": round(algorithmic_bytes(m, n, k) / us / 1e3, 1),
@@ -277,7 +283,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=200, help="untimed launches directly before the timed ones")
-    ap.add_argument("--config", default=None, choices=sorted(CONFIGS),
+    ap.add_argument("--config", default=None, choices=sorted(CONFIGS) + sorted(EXTRA_CONFIGS),
                     help="run only this configuration (default: C2 as the headline plus all_configs)")
     ap.add_argument("--all", action="store_true", help="also quantisers, grouped form, operand bits, MFMA ceiling")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity gate")
@@ -302,7 +308,7 @@ def main():
     stream = torch.cuda.Stream()
 
     headline = args.config or "C2"
-    m, n, k, seed = CONFIGS[headline]
+    m, n, k, seed = {**CONFIGS, **EXTRA_CONFIGS}[headline]
     rec, data, g, gen_s, us_burst, cpu_s = measure_config(rfk, cref, rk, headline, args.steps, args.warmup, stream,
                                                           not args.no_cpu, args.settle, keep=True)
     us = rec["us_per_gemm"]
