@@ -48,7 +48,7 @@ EXTRA_CONFIGS = {
 }
 RTOL, ATOL, ATOL_REFERENCE = 2e-2, 1e-2, 1e-3
 SETTLE_SECONDS = 0.4
-KERNEL_SOURCES = ("fp8_gemm_kernels.h", "fp8_gemm_persistent.h")
+KERNEL_SOURCES = ("fp8_gemm_kernels.h", "fp8_gemm_persistent.h", "fp8_gemm_skinny.h", "gemm_launcher.hip")
 
 
 def kernel_source_sha():
@@ -245,7 +245,7 @@ def measure_config(rfk, cref, rk, name, steps, warmup, stream, with_cpu, settle_
     us, settle = settled_us(rfk, g, steps, warmup, settle_seconds)
     cfg = rfk.select_config(m, n, k)
     schedule = {0: "gemm_fp8_blockscale_tile", 1: "gemm_fp8_blockscale_streamk", 2: "gemm_fp8_blockscale_persistent",
-                3: "gemm_fp8_blockscale_persistent with a last round of half tiles"}
+                3: "gemm_fp8_blockscale_persistent with a last round of half tiles", 4: "gemm_fp8_blockscale_skinny"}
     launches = 1 if cfg.split_k == 1 else 2
     rec = {"shape": [m, n, k], "us_per_gemm": round(us, 2), "settle_launches": settle,
            "tflops": round(2.0 * m * n * k / us / 1e6, 1), "gbs_algorithmic": round(algorithmic_bytes(m, n, k) / us / 1e3, 1),

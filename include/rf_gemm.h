@@ -45,7 +45,8 @@ enum {
     RF_ERR_BAD_CONFIG = 4      /* explicit config not available for this shape */
 };
 
-enum { RF_SCHEDULE_TILES = 0, RF_SCHEDULE_STREAM_K = 1, RF_SCHEDULE_PERSISTENT = 2, RF_SCHEDULE_PERSISTENT_HALF_TAIL = 3 };
+enum { RF_SCHEDULE_TILES = 0, RF_SCHEDULE_STREAM_K = 1, RF_SCHEDULE_PERSISTENT = 2, RF_SCHEDULE_PERSISTENT_HALF_TAIL = 3,
+       RF_SCHEDULE_SKINNY_K = 4 };
 
 /* One launch plan: which kernel variant and how K is split.
  * Replaces a DISPATCH_GEMM(...) line of the reference (src/gemm/gemm_launcher.cpp:158-162,229-259). */
@@ -63,7 +64,11 @@ typedef struct rf_gemm_config {
                          3 PERSISTENT_HALF_TAIL  the persistent schedule for the whole rounds of one tile per CU, the
                                       left-over tiles finished as 128-row half tiles, one per CU; 256x256 tile only,
                                       needs the persistent schedule's shape rules, at least one tile per CU and a
-                                      last round that is at most half full */
+                                      last round that is at most half full;
+                         4 SKINNY_K   K = 128 or 256 only: persistent grid, a workgroup keeps the B operand of a strip of
+                                      256 columns in registers and streams A in items of 128 rows, storing each
+                                      16-row piece of C as soon as it is complete (the launch is a streaming store of
+                                      C); needs variant == 0, split_k == 1, M a multiple of 16, N a multiple of 64 */
 } rf_gemm_config;
 
 /* Drop-in for the reference's launcher entry (src/gemm/gemm_launcher.cpp:182-184):

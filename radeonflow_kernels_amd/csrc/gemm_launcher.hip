@@ -18,6 +18,7 @@
 #include "../../include/rf_gemm.h"
 #include "fp8_gemm_kernels.h"
 #include "fp8_gemm_persistent.h"
+#include "fp8_gemm_skinny.h"
 #include "quantize_kernels.h"
 
 // Scratch memory of rf_fp8_gemm_static, the entry point that allocates nothing: split-K partial sums and staging
@@ -170,7 +171,7 @@ int parse_plans(const char *path, std::vector<TunedPlan> &out) {
         if (got <= 0) continue;                       // blank or comment line
         if (got != 7 || p.m < 1 || p.n < 1 || p.k < rf::BK || p.k % rf::BK != 0 || p.variant < 0 ||
             p.variant >= kNumVariants || p.split_k < 1 || p.group_m < 1 || p.stream_k < RF_SCHEDULE_TILES ||
-            p.stream_k > RF_SCHEDULE_PERSISTENT_HALF_TAIL || (p.stream_k != RF_SCHEDULE_TILES && p.split_k != 1)) {
+            p.stream_k > RF_SCHEDULE_SKINNY_K || (p.stream_k != RF_SCHEDULE_TILES && p.split_k != 1)) {
             fclose(f);
             return fail(RF_ERR_BAD_CONFIG, std::string(path) + ":" + std::to_string(lineno) +
                                                ": expected \"M N K variant split_k group_m stream_k\" with valid values");
@@ -211,6 +212,10 @@ int ensure_device_info(State &s) {
             RF_HIP(hipFuncSetAttribute((const void *)v.persistent_half_tail, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        v.lds_persistent));
     }
+    RF_HIP(hipFuncSetAttribute((const void *)rf::gemm_fp8_blockscale_skinny<1>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                               rf::SkinnyGeom<1>::LDS_BYTES));
+    RF_HIP(hipFuncSetAttribute((const void *)rf::gemm_fp8_blockscale_skinny<2>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                               rf::SkinnyGeom<2>::LDS_BYTES));
     // the device address of this device's copy of the scratch array (the array's name is only a host-side handle)
     void *scratch_ptr = nullptr;
     RF_HIP(hipGetSymbolAddress(&scratch_ptr, HIP_SYMBOL(scratch)));
@@ -350,6 +355,11 @@ bool half_tail_ok(const Variant &v, int m, int n, int k, int num_cu) {
     return t >= num_cu && r > 0 && (r + 7) / 8 * 8 + r <= num_cu;
 }
 
+// Skinny-K schedule (fp8_gemm_skinny.h): one or two K blocks, whole 16-row m-tiles and whole 64-column wave tiles.
+bool skinny_ok(int m, int n, int k) {
+    return (k == rf::BK || k == 2 * rf::BK) && m >= 16 && m % 16 == 0 && n >= 64 && n % 64 == 0;
+}
+
 // Stream-K: at least one tile per workgroup (then a split tile has exactly two contributors, which is all the kernel
 // handles) and no more tiles than arrival counters.
 bool stream_k_ok(const Variant &v, int m, int n, int num_cu) {
@@ -379,7 +389,8 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
         return p.m == m && p.n == n && p.k == k && p.variant < kNumVariants && p.split_k <= k / rf::BK &&
                (p.stream_k != RF_SCHEDULE_PERSISTENT || persistent_ok(kVariants[p.variant], m, n, k)) &&
                (p.stream_k != RF_SCHEDULE_STREAM_K || stream_k_ok(kVariants[p.variant], m, n, num_cu)) &&
-               (p.stream_k != RF_SCHEDULE_PERSISTENT_HALF_TAIL || half_tail_ok(kVariants[p.variant], m, n, k, num_cu));
+               (p.stream_k != RF_SCHEDULE_PERSISTENT_HALF_TAIL || half_tail_ok(kVariants[p.variant], m, n, k, num_cu)) &&
+               (p.stream_k != RF_SCHEDULE_SKINNY_K || skinny_ok(m, n, k));
     };
     const TunedPlan *hit = nullptr;
     for (const TunedPlan &p : user_plans)
@@ -391,6 +402,15 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
         out->split_k = hit->split_k;
         out->group_m = hit->group_m;
         out->stream_k = hit->stream_k;
+        return;
+    }
+    // One or two K blocks and a large C: the launch is a streaming store, which the skinny-K schedule does best
+    // (measured against the best tiled plan at N = 7168, K = 256: 1024 rows 6.5 against 6.9 us, 2048 rows 7.8 against
+    // 10.3, 6144 rows 18.2 against 22.1; below about six million outputs the 64 x 128 tiles win, e.g. 2048 x 2048: 6.5
+    // against 5.6 us).
+    if (skinny_ok(m, n, k) && (double)m * n >= 6.0e6) {
+        out->variant = 0;
+        out->stream_k = RF_SCHEDULE_SKINNY_K;
         return;
     }
     // No measured entry: a cost model fitted to the tuner's measurements of the tabled shapes (on those
@@ -472,6 +492,9 @@ int launch_locked(State &s, Mem &mem, const void *a, const void *b, const float 
                 return fail(RF_ERR_BAD_CONFIG, "the half-tile schedule needs the 256x256 tile, the persistent schedule's "
                                                "shape rules, at least one tile per compute unit and a last round that "
                                                "is at most half full");
+        } else if (cfg.stream_k == RF_SCHEDULE_SKINNY_K) {
+            if (cfg.variant != 0 || !skinny_ok(m, n, k))
+                return fail(RF_ERR_BAD_CONFIG, "the skinny-K schedule needs variant 0, K = 128 or 256, M a multiple of 16 and N a multiple of 64");
         } else if (cfg.stream_k != RF_SCHEDULE_TILES) {
             return fail(RF_ERR_BAD_CONFIG, "unknown schedule");
         }
@@ -506,6 +529,23 @@ int launch_locked(State &s, Mem &mem, const void *a, const void *b, const float 
         hipLaunchKernelGGL(v.persistent, dim3(T < P ? T : P), block, v.lds_persistent, stream,
                            (const uint8_t *)a, (const uint8_t *)b, as, bs, (uint16_t *)c, m, n, k, tiles_m, tiles_n,
                            cfg.group_m, m_store);
+        RF_HIP(hipGetLastError());
+        return RF_OK;
+    }
+    if (cfg.stream_k == RF_SCHEDULE_SKINNY_K) {
+        // one strip of 256 columns per workgroup, and as many workgroups per strip as fill the chip once (each takes a
+        // share of the strip's rows, in units of 64)
+        const int strips = ceil_div(n, 256), units = ceil_div(m, 64);
+        int per_strip = s.num_cu / strips;
+        per_strip = per_strip < 1 ? 1 : per_strip > units ? units : per_strip;
+        if (qk == 1)
+            hipLaunchKernelGGL(rf::gemm_fp8_blockscale_skinny<1>, dim3(strips * per_strip), dim3(512),
+                               rf::SkinnyGeom<1>::LDS_BYTES, stream, (const uint8_t *)a, (const uint8_t *)b, as, bs,
+                               (uint16_t *)c, m, n, per_strip, m_store);
+        else
+            hipLaunchKernelGGL(rf::gemm_fp8_blockscale_skinny<2>, dim3(strips * per_strip), dim3(512),
+                               rf::SkinnyGeom<2>::LDS_BYTES, stream, (const uint8_t *)a, (const uint8_t *)b, as, bs,
+                               (uint16_t *)c, m, n, per_strip, m_store);
         RF_HIP(hipGetLastError());
         return RF_OK;
     }

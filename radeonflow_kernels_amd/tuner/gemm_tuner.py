@@ -78,17 +78,19 @@ def tune_shape(rfk, m, n, k, log=print):
     for v in rfk.variants():
         tiles = -(-m // v["block_m"]) * -(-n // v["block_n"])
         # schedules: 0 = one workgroup per tile (with K splits), 1 = stream-K, 2 = persistent whole tiles,
-        # 3 = persistent with a last round of half tiles
-        for split, sk in [(sp, 0) for sp in SPLITS] + [(1, 1), (1, 2), (1, 3)]:
+        # 3 = persistent with a last round of half tiles, 4 = skinny K (K = 128 or 256; listed under variant 0)
+        for split, sk in [(sp, 0) for sp in SPLITS] + [(1, 1), (1, 2), (1, 3), (1, 4)]:
             if split > k // 128 or (sk == 1 and (tiles < ncu or not v["stream_k"])):
                 continue
             if sk in (2, 3) and (not v["persistent"] or m < v["block_m"] or m % 16 or n % v["block_n"] or (k // 128) % 2):
+                continue
+            if sk == 4 and (v["variant"] != 0 or k > 256 or m % 16 or n % 64):
                 continue
             if sk == 3:
                 left = tiles % ncu
                 if v["variant"] != 0 or tiles < ncu or left == 0 or (left + 7) // 8 * 8 + left > ncu:
                     continue
-            for gm in GROUPS:
+            for gm in (GROUPS if sk != 4 else GROUPS[1:2]):          # the skinny-K schedule has no tile order to group
                 cfg = rfk.GemmConfig(v["variant"], split, gm, sk)
                 args[4].zero_()
                 us = _time(rfk, args, cfg, iters)

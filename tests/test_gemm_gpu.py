@@ -191,12 +191,13 @@ def test_ragged_m_under_a_persistent_plan_writes_c_in_place(rfk, tmp_path):
         rfk.clear_plans()
 
 
-@pytest.mark.parametrize("m", [6000, 6001])
-def test_large_m_that_is_not_a_tile_multiple_runs_the_persistent_plan_automatically(rfk, m):
-    """6000 and 6001 rows with C4's N and K: the automatic plan is the persistent schedule (for 6001 on the shape padded
-    to 6016 rows, with C written in place); exact data, bit for bit, canary behind the last true row intact."""
-    n, k = 7168, 256
-    assert rfk.select_config(m, n, k).stream_k == 2
+@pytest.mark.parametrize("m,k,schedule", [(6000, 512, 2), (6001, 512, 2), (6000, 256, 4), (6001, 256, 4)])
+def test_large_m_that_is_not_a_tile_multiple_runs_a_whole_tile_plan_automatically(rfk, m, k, schedule):
+    """6000 and 6001 rows with C4's N: the automatic plan is the persistent schedule at K = 512 and the skinny-K schedule
+    at K = 256 (for 6001 on the shape padded to 6016 rows, with C written in place: both schedules mask the padding
+    rows in their stores); exact data, bit for bit, canary behind the last true row intact."""
+    n = 7168
+    assert rfk.select_config(m, n, k).stream_k == schedule
     data = exact_problem(m, n, k, seed=m)
     out = _run(rfk, data, canary=8192)
     assert np.array_equal(bf16_bits(out), oracle_bf16(data))
@@ -253,6 +254,34 @@ def test_half_tile_schedule_rejects_shapes_it_does_not_fit(rfk):
         data = exact_problem(m, n, k, seed=1)
         with pytest.raises(RuntimeError):
             _run(rfk, data, config=rfk.GemmConfig(variant, 1, 8, 3))
+
+
+@pytest.mark.parametrize("m,n,k", [(128, 256, 256), (16, 64, 128), (272, 320, 256), (1040, 448, 128), (2048, 2048, 256),
+                                   (6000, 7168, 256), (96, 7168, 256), (400, 1216, 256)])
+def test_skinny_k_schedule_bit_exact(rfk, m, n, k):
+    """K = 128 or 256 under the skinny-K schedule (the B operand of a 256-column strip in registers, A streamed in
+    items of 128 rows, C stored m-tile by m-tile): strips that end in a partial 64-column wave tile, a last item with
+    fewer than 128 rows, one to many items and strips per workgroup. Exact data against the oracle, bit for bit, twice
+    on the same buffers with the canary intact; then data with rounding in it against the one-workgroup-per-tile
+    kernel, bit for bit as well (same MFMA, same folds in the same K order)."""
+    cfg = rfk.GemmConfig(0, 1, 8, 4)
+    data = exact_problem(m, n, k, seed=m + n + k)
+    exp = oracle_bf16(data)
+    for rep in range(2):
+        out = _run(rfk, data, config=cfg, canary=1024)
+        assert np.array_equal(bf16_bits(out), exp), "rep %d" % rep
+    noisy = rk.generate_input_blockquant(m, n, k, seed=m + k)
+    ref = bf16_bits(_run(rfk, noisy, config=rfk.GemmConfig(1, 1, 8, 0))).copy()
+    out = _run(rfk, noisy, config=cfg, canary=1024)
+    assert np.array_equal(bf16_bits(out), ref)
+    assert_close_to_oracle(out, oracle_bf16(noisy), RTOL, ATOL, "skinny K")
+
+
+def test_skinny_k_schedule_rejects_shapes_it_does_not_fit(rfk):
+    for (m, n, k, variant) in ((256, 256, 384, 0), (256, 256, 512, 0), (40, 256, 256, 0), (256, 96, 256, 0), (256, 256, 256, 1)):
+        data = exact_problem(m, n, k, seed=1)
+        with pytest.raises(RuntimeError):
+            _run(rfk, data, config=rfk.GemmConfig(variant, 1, 8, 4))
 
 
 def test_persistent_schedule_rejects_ragged_shapes(rfk):
