@@ -5,7 +5,10 @@
 //   +folds      every MFMA starts from zero and its result is folded into one of 32 accumulator tiles with four
 //               fp32 FMAs three slots later, as the block-scaled GEMM must (scale * partial + acc);
 //   +lds_reads  in addition the operand fragments are re-read from LDS with ds_read_b64_tr_b8 at the GEMM's rate
-//               (28 + 16 transpose reads per 32 MFMAs, conflict-free layout), still without any global memory traffic.
+//               (28 + 16 transpose reads per 32 MFMAs, conflict-free layout), still without any global memory traffic;
+//   +b128_reads the same fragments read from a K-contiguous LDS layout instead (a row = one m or n, 128 bytes of K, 16-byte
+//               chunks XOR-swizzled by row): two ds_read_b128 per fragment, half as many LDS instructions for the same
+//               bytes. Prices operands that arrive K-contiguous (prepacked weights, a quantiser that writes them so).
 // The published peak (5.0 PFLOP/s dense) assumes 2.4 GHz; under load the chip lowers its clock to stay inside its
 // power limit, and how far depends on how many bits toggle in the operands and on what else the loop executes.
 // The "+lds_reads" figure for realistic operands is the ceiling a block-scaled fp8 GEMM with fp32 folds on the vector
@@ -13,7 +16,8 @@
 //
 //   mfma_ceiling [seconds per mode] [compute units]     prints one JSON line:
 //   {"zeros": T, "normal": T, "random_bits": T, "normal_with_folds": T, "normal_with_folds_and_lds_reads": T,
-//    "zeros_with_folds_and_lds_reads": T, "unit": "TFLOP/s", "cus": n, "implied_clock_ghz": {...}}
+//    "normal_with_folds_and_b128_reads": T, "zeros_with_folds_and_lds_reads": T, "unit": "TFLOP/s", "cus": n,
+//    "implied_clock_ghz": {...}}
 // zeros: all operand bytes 0. normal: e4m3fn codes of N(0,1) samples scaled so that 4.5 sigma maps to 448 (what a
 // blockwise quantiser produces). random_bits: uniformly random finite e4m3fn codes. With fewer compute units than the
 // chip has (second argument) the power limit is out of the picture and the figures show the cost in cycles alone.
@@ -36,6 +40,9 @@ constexpr int kWords = 4096, kSlots = 32, kLdsBytes = 32768;
 // MODE 0: acc = mfma(a, b, acc). MODE 1: p = mfma(a, b, 0); acc[t] = fma(s, p three slots ago, acc[t]).
 // MODE 2: MODE 1 + the fragments re-read from LDS (a 128-row K block of 256-byte rows, 16-byte chunks XOR-swizzled by
 // row like the GEMM's stages, so that the transpose reads are free of bank conflicts).
+// MODE 3: MODE 1 + the fragments re-read with ds_read_b128 from a K-contiguous layout (256 rows of 128 bytes; lane (L, g)
+// takes bytes 32 g .. 32 g + 31 of row L of the fragment's 16 rows; chunk index XORed with (row >> 1) & 7, so that the
+// 16 lanes the LDS serves together touch 16 different 16-byte bank groups).
 template <int MODE>
 __global__ __launch_bounds__(512) void inner_loop(const int *__restrict__ src, float *out, int iters, float sc) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
@@ -56,6 +63,28 @@ __global__ __launch_bounds__(512) void inner_loop(const int *__restrict__ src, f
     const uint32_t off = krow * 256 + 8 * (L & 1);
     auto rd = [&](int chunk, int t) {
         return __builtin_amdgcn_ds_read_tr8_b64_v2i32((RF_LDS i32x2 *)(lds + off + (((chunk & 15) ^ swz) << 4) + t * 2048));
+    };
+    typedef int i32x4 __attribute__((ext_vector_type(4)));
+    auto rd128 = [&](int frag, int h) {
+        const int row = (16 * frag + L) & 255, chunk = (2 * g + h) ^ ((L >> 1) & 7);
+        return *(RF_LDS i32x4 *)(lds + row * 128 + chunk * 16);
+    };
+    auto reread128 = [&](int t) {        // the same fragments at the same slots, two 16-byte reads each
+        if (t % 4 == 0 && t < 28) {
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const i32x4 v = rd128(t / 4, h);
+#pragma unroll
+                for (int e = 0; e < 4; e++) a[((t / 4) + 1) & 1][4 * h + e] = v[e];
+            }
+        } else if (t >= 28) {
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const i32x4 v = rd128(8 + t, h);
+#pragma unroll
+                for (int e = 0; e < 4; e++) b[t - 28][4 * h + e] = v[e];
+            }
+        }
     };
     auto reread = [&](int t) {           // the GEMM's pattern: next m-tile's fragment, then the next block's fragments
         if (t % 4 == 0 && t < 28) {
@@ -100,6 +129,7 @@ __global__ __launch_bounds__(512) void inner_loop(const int *__restrict__ src, f
                 asm volatile("" : "+v"(pr[t % 4]));
                 __builtin_amdgcn_sched_barrier(0);
                 if constexpr (MODE == 2) reread(t);
+                if constexpr (MODE == 3) reread128(t);
                 const int u = (t + kSlots - 3) % kSlots;
 #pragma unroll
                 for (int e = 0; e < 4; e++) acc[u][e] = __builtin_fmaf(s[u / 4], pr[u % 4][e], acc[u][e]);
@@ -155,9 +185,10 @@ int main(int argc, char **argv) {
     // (operand bits, loop form): the three operand kinds on the bare MFMA loop, then the GEMM's extra work
     const struct { int data, loop; const char *key; } runs[] = {
         {0, 0, "zeros"}, {1, 0, "normal"}, {2, 0, "random_bits"}, {1, 1, "normal_with_folds"},
-        {1, 2, "normal_with_folds_and_lds_reads"}, {0, 2, "zeros_with_folds_and_lds_reads"}};
+        {1, 2, "normal_with_folds_and_lds_reads"}, {1, 3, "normal_with_folds_and_b128_reads"},
+        {0, 2, "zeros_with_folds_and_lds_reads"}};
     constexpr int kRuns = sizeof(runs) / sizeof(runs[0]);
-    const kernel_t kernels[3] = {inner_loop<0>, inner_loop<1>, inner_loop<2>};
+    const kernel_t kernels[4] = {inner_loop<0>, inner_loop<1>, inner_loop<2>, inner_loop<3>};
     double tflops[kRuns], ghz[kRuns];
     for (int r = 0; r < kRuns; r++) {
         std::mt19937 data_rng(1);

@@ -19,8 +19,13 @@
  * Temporary device memory (split-K partial sums, staging copies, stream-K counters) is kept per (device, stream), for
  * the device that is current at the call: launches on different streams of one device may overlap, launches on one
  * stream are ordered by the stream. Calls are serialised by one lock only while they enqueue. A buffer that has to grow
- * is replaced and the old one freed by rf_gemm_destroy, so no call waits for the device (up to 32 streams per device
- * have a buffer set of their own; a caller that cycles through more pays a device-wide wait when a set changes hands).
+ * is replaced and the old one freed by rf_gemm_destroy, so no call waits for the device. A stream gets a buffer set only
+ * when a launch on it needs temporary memory (most plans need none); up to 32 streams per device have a set of their
+ * own, and when one more asks, the least recently used set changes hands: the new stream waits on the device for the
+ * old stream's work enqueued so far (an event, no host wait). A stream that is being captured into a HIP graph cannot
+ * take a set over and gets RF_ERR_BAD_CONFIG (its first 32 streams capture fine; rf_fp8_gemm_static never needs a set).
+ * HIP graphs captured through this library refer to these buffers: destroy them before rf_gemm_destroy, and do not
+ * replay a graph captured on a stream whose set has since changed hands.
  */
 #ifndef RF_GEMM_H
 #define RF_GEMM_H
@@ -75,7 +80,11 @@ typedef struct rf_gemm_config {
  * same name, argument order and behaviour: enqueues on job_stream0 and returns; on any error prints a
  * message and abort()s (src/gemm/gemm_launcher.cpp:96-100,261-264). metrics may be NULL; if not,
  * entries[0].time (ms) and entries[0].gflops are written from a stream callback once the work has
- * finished (src/utils/timer.cpp:12-60). */
+ * finished (src/utils/timer.cpp:12-60). Like the reference's, the callback reads the two events with
+ * hipEventElapsedTime, a call HIP does not promise to allow inside a stream callback (the ROCm runtime this library is
+ * built for does); it is the only way to have the figures written before a hipDeviceSynchronize() that follows run()
+ * returns, which is what the reference's checker relies on (tests/checker/checker.cpp:286-336). Pass metrics = NULL
+ * (or call rf_fp8_gemm) to keep callbacks out of the stream altogether. */
 void run(void *a, void *b, void *as, void *bs, void *c, int m, int n, int k, PerfMetrics *metrics,
          hipStream_t job_stream0);
 
@@ -86,13 +95,18 @@ int rf_fp8_gemm(const void *a, const void *b, const float *as, const float *bs, 
 
 /* rf_fp8_gemm for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc. No counterpart in the reference (its launcher allocates a fixed workspace with
- * hipMalloc on first use, src/gemm/gemm_launcher.cpp:30-36). Same arguments, plan choice and result bits as
- * rf_fp8_gemm, but split-K partial sums and the staging copies of ragged or unaligned operands live in a static
- * device array of rf_gemm_static_scratch_bytes() bytes (32 MiB; every GPU the library has run on holds one until the
- * process ends), and the call allocates and frees nothing. A shape whose plan needs more scratch memory than that
- * fails with RF_ERR_BAD_CONFIG (rf_gemm_last_error() gives the bytes needed), as does a stream-K plan from a plan
- * file. All calls on one GPU share that GPU's array: two calls that overlap in time (different streams, or graph
- * replays beside eager launches) race; calls on one stream are ordered by the stream. */
+ * hipMalloc on first use, src/gemm/gemm_launcher.cpp:30-36). Same arguments as rf_fp8_gemm, but split-K partial sums
+ * and the staging copies of ragged or unaligned operands live in a static device array of
+ * rf_gemm_static_scratch_bytes() bytes (32 MiB; every GPU the library has run on holds one until the process ends),
+ * and the call allocates and frees nothing. The plan is rf_fp8_gemm's, and so are the result bits, whenever that plan
+ * fits the array. Otherwise the plan is fitted to it: a K split is cut down to as many parts as fit (one part needs no
+ * scratch memory), a stream-K plan from a plan file is replaced by the automatic plan, and a ragged or unaligned shape
+ * whose staging copies do not fit as a whole is computed in row ranges that take turns in the array (M = 6001, N = 4608,
+ * K = 7168: two ranges); such results agree with rf_fp8_gemm's within the rounding of another K split, and bit for bit
+ * on data whose sums are exact. Only when the staged copy of B (ragged N or an unaligned b) alone takes more than half
+ * of the array does the much slower bounds-checked kernel compute the shape, in place. All calls on one GPU share that
+ * GPU's array: two calls that overlap in time (different streams, or graph replays beside eager launches) race; calls on
+ * one stream are ordered by the stream. */
 int rf_fp8_gemm_static(const void *a, const void *b, const float *as, const float *bs, void *c,
                        int m, int n, int k, hipStream_t stream);
 size_t rf_gemm_static_scratch_bytes(void);
@@ -112,6 +126,12 @@ int rf_fp8_gemm_time(const void *a, const void *b, const float *as, const float 
 /* The plan rf_fp8_gemm would use for (m,n,k) on the current device: the gfx950 replacement of the
  * per-shape table in src/gemm/gemm_launcher.cpp:229-259 / tuner/gemm_tuner.py. */
 int rf_gemm_select_config(int m, int n, int k, rf_gemm_config *out);
+
+/* The plan for (m,n,k) on a device with num_cu compute units, worked out on the host alone (no device is touched, the
+ * file named by RF_GEMM_PLANS is not read; plans loaded with rf_gemm_load_plans count). The built-in table was measured
+ * on 256 compute units and is consulted only for that count; any other count gets the cost model, which counts rounds
+ * of workgroups for the count given. For capacity planning and for tests of the planner's arithmetic. */
+int rf_gemm_plan_for(int m, int n, int k, int num_cu, rf_gemm_config *out);
 
 /* Measured plans from a file, looked up before the built-in table (the role of pasting DISPATCH_GEMM lines into the
  * reference's launcher, src/gemm/gemm_launcher.cpp:229-259, tuner/gemm_batch.py:196-200, without a rebuild). One plan

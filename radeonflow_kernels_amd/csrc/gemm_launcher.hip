@@ -243,11 +243,16 @@ hipError_t device_malloc(void **p, size_t bytes) {
 // Where a launch finds its temporary device memory: the growable buffers of its (device, stream), or, for
 // rf_fp8_gemm_static, consecutive pieces of the device's static scratch array (nothing is allocated; a launch that
 // needs more than the array holds fails).
+int buffers_of(State &s, hipStream_t stream, StreamBuffers **out);
 struct Mem {
     State &s;
-    StreamBuffers *sb = nullptr;         // growable buffers (null in static mode)
+    StreamBuffers *sb = nullptr;         // growable buffers of `stream`, bound at the first use (never in static mode)
     uint8_t *fixed = nullptr;            // static mode: this device's scratch array
     size_t fixed_used = 0;
+    hipStream_t stream = nullptr;
+    // Most launches need no temporary memory at all (one kernel, no K split, no staging): the stream's buffer set is
+    // looked up, and past kMaxStreamBuffers streams taken over from another stream, only when a buffer is asked for.
+    int bind() { return sb ? RF_OK : buffers_of(s, stream, &sb); }
 
     template <typename T>
     int grow(T *&buf, size_t &have, size_t need) {
@@ -271,27 +276,46 @@ struct Mem {
         fixed_used = at + bytes;
         return RF_OK;
     }
+    // bytes the static array still has to give (after rounding the next piece up to 256)
+    size_t fixed_left() const {
+        const size_t at = (fixed_used + 255) / 256 * 256;
+        return at < kStaticScratchBytes ? kStaticScratchBytes - at : 0;
+    }
     int pad(size_t bytes, uint8_t **out) {
         if (fixed) return take_fixed(bytes, (void **)out, "staging copy of ragged or unaligned operands");
-        int rc = grow(sb->pad, sb->pad_bytes, bytes);
+        int rc = bind();
+        if (rc != RF_OK) return rc;
+        rc = grow(sb->pad, sb->pad_bytes, bytes);
         *out = sb->pad;
         return rc;
     }
     int workspace(size_t bytes, float **out) {
         if (fixed) return take_fixed(bytes, (void **)out, "split-K partial sums");
-        int rc = grow(sb->ws, sb->ws_bytes, bytes);
+        int rc = bind();
+        if (rc != RF_OK) return rc;
+        rc = grow(sb->ws, sb->ws_bytes, bytes);
         *out = sb->ws;
         return rc;
     }
     int tile_counters(unsigned **out) {
         if (fixed) return fail(RF_ERR_BAD_CONFIG, "rf_fp8_gemm_static: the stream-K schedule is not available");
+        int rc = bind();
+        if (rc != RF_OK) return rc;
         if (!sb->tile_count) RF_HIP(device_malloc((void **)&sb->tile_count, kMaxStreamKTiles * sizeof(unsigned)));
         if (!sb->tile_count_zeroed) {
             // zeroed on the stream of the launch that follows (the kernels leave the counters at zero afterwards);
             // a kernel and not a memset, so that the call may be recorded into a HIP graph. A recorded fill has not
             // run yet, so it does not count: launches keep filling first until one has done so for real.
+            // (on the legacy null stream the query itself is refused while another thread captures in global mode:
+            // that counts as "capturing", so the fill is issued and the flag stays false)
             hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
-            RF_HIP(hipStreamIsCapturing(sb->stream, &st));
+            const hipError_t qe = hipStreamIsCapturing(sb->stream, &st);
+            if (qe == hipErrorStreamCaptureImplicit || qe == hipErrorStreamCaptureUnsupported) {
+                (void)hipGetLastError();
+                st = hipStreamCaptureStatusActive;
+            } else if (qe != hipSuccess) {
+                return fail(RF_ERR_HIP, std::string("hipStreamIsCapturing: ") + hipGetErrorString(qe));
+            }
             hipLaunchKernelGGL(zero_words, dim3(kMaxStreamKTiles / 256), dim3(256), 0, sb->stream, sb->tile_count);
             RF_HIP(hipGetLastError());
             sb->tile_count_zeroed = st == hipStreamCaptureStatusNone;
@@ -302,8 +326,10 @@ struct Mem {
 };
 
 // The buffer set of (current device, stream); the caller holds the lock. A set prepared by rf_gemm_init and not yet
-// bound to a stream is taken first. Past kMaxStreamBuffers streams the least recently used set changes hands, after
-// a device-wide wait (the only host wait in the launch path, and only for callers that cycle through that many streams).
+// bound to a stream is taken first. Past kMaxStreamBuffers streams the least recently used set changes hands: the new
+// stream is made to wait (on the device, through an event) for what the old stream has enqueued so far, so the host
+// does not wait. A stream that is being captured into a graph cannot take a set over (the wait would become part of
+// the graph, and the old stream's later work would not be ordered against the graph's replays): RF_ERR_BAD_CONFIG.
 constexpr uintptr_t kUnboundStream = 1;  // not a valid stream handle
 int buffers_of(State &s, hipStream_t stream, StreamBuffers **out) {
     StreamBuffers *unbound = nullptr, *lru = nullptr;
@@ -323,7 +349,24 @@ int buffers_of(State &s, hipStream_t stream, StreamBuffers **out) {
         b = &s.buffers.back();
     }
     if (!b) {
-        RF_HIP(hipDeviceSynchronize());
+        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+        const hipError_t qe = hipStreamIsCapturing(stream, &st);
+        if (qe != hipSuccess || st != hipStreamCaptureStatusNone) {
+            if (qe != hipSuccess) (void)hipGetLastError();
+            return fail(RF_ERR_BAD_CONFIG, "more than " + std::to_string(kMaxStreamBuffers) + " streams have used temporary "
+                        "device memory on this device, and a stream that is being captured cannot take over another "
+                        "stream's buffers: use rf_fp8_gemm_static under capture, or fewer streams");
+        }
+        hipEvent_t ev = nullptr;
+        RF_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+        hipError_t e = hipEventRecord(ev, lru->stream);
+        if (e == hipSuccess) e = hipStreamWaitEvent(stream, ev, 0);
+        (void)hipEventDestroy(ev);                               // released once the wait has been satisfied
+        if (e != hipSuccess) {
+            // the old stream no longer exists (or is being captured): wait for the device instead
+            (void)hipGetLastError();
+            RF_HIP(hipDeviceSynchronize());
+        }
         b = lru;
     }
     b->stream = stream;
@@ -375,6 +418,8 @@ const TunedPlan kTunedPlans[] = {
 #include "tuned_plans.inc"
 };
 
+constexpr int kTunedOnCUs = 256;
+
 // Heuristic plan for shapes without a measured entry. Inputs: shape and CU count.
 void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::vector<TunedPlan> &user_plans,
                    rf_gemm_config *out) {
@@ -395,8 +440,12 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
     const TunedPlan *hit = nullptr;
     for (const TunedPlan &p : user_plans)
         if (!hit && usable(p)) hit = &p;
-    for (const TunedPlan &p : kTunedPlans)
-        if (!hit && usable(p)) hit = &p;
+    // the compiled-in table was measured on a device with kTunedOnCUs compute units: round counts, and with them the
+    // best tile and split, change with the unit count, so another device takes the cost model below (which counts
+    // rounds for the device at hand) unless the caller has loaded plans measured there
+    if (num_cu == kTunedOnCUs)
+        for (const TunedPlan &p : kTunedPlans)
+            if (!hit && usable(p)) hit = &p;
     if (hit) {
         out->variant = hit->variant;
         out->split_k = hit->split_k;
@@ -502,6 +551,19 @@ int launch_locked(State &s, Mem &mem, const void *a, const void *b, const float 
         select_config(m, n, k, s.num_cu, tiled_ok, shared().user_plans, &cfg);
     }
 
+    if (mem.fixed && cfg.variant >= 0) {
+        // rf_fp8_gemm_static: the plan has to live inside what is left of the static array. A stream-K plan (only a
+        // plan file can name one) is replaced by the cost model's plan; a K split whose partial sums do not fit is cut
+        // down to the number of parts that do, a single part needing no scratch memory at all.
+        if (cfg.stream_k == RF_SCHEDULE_STREAM_K) select_config(m, n, k, s.num_cu, true, std::vector<TunedPlan>(), &cfg);
+        if (cfg.stream_k == RF_SCHEDULE_STREAM_K) cfg.stream_k = RF_SCHEDULE_TILES;
+        if (cfg.split_k > 1) {
+            const size_t per_part = (size_t)m * n * sizeof(float);
+            const int qk_ = k / rf::BK, kb_per = ceil_div(qk_, cfg.split_k), parts = ceil_div(qk_, kb_per);
+            const size_t fit = mem.fixed_left() / per_part;
+            if ((size_t)parts > fit) cfg.split_k = fit < 2 ? 1 : (int)fit;
+        }
+    }
     if (m_store != m && (cfg.variant < 0 || cfg.stream_k == RF_SCHEDULE_STREAM_K))
         return fail(RF_ERR_BAD_CONFIG, "internal: this schedule cannot write fewer rows than it computes");
     if (cfg.variant < 0) {
@@ -715,6 +777,66 @@ rf::GroupTable one_group(int cols, int cols_pad) {
     return t;
 }
 
+// rf_fp8_gemm_static on a ragged or unaligned shape whose staging copies do not fit the static array as a whole: the
+// rows of the problem are cut into pieces (row ranges of A, a_scale and C are independent GEMMs), each piece is staged,
+// computed and, where C is staged too, copied back before the next one re-uses the same memory; the stream orders them.
+// The staged copy of B (ragged N or an unaligned b) is shared by all pieces and has to fit beside them: when it takes
+// more than half of the array, the bounds-checked kernel computes the whole problem in place instead.
+int launch_padded_in_pieces(State &s, Mem &mem, const void *a, const void *b, const float *as, const float *bs, void *c,
+                            int m, int n, int k, hipStream_t stream) {
+    auto pad16 = [](int x) { return x < 16 ? 16 : (x + 15) / 16 * 16; };
+    auto align = [](size_t x) { return (x + 255) / 256 * 256; };
+    const int np = pad16(n), qk = k / rf::BK;
+    const bool copy_b = np != n || (uintptr_t)b % 16 != 0;
+    const bool copy_c = np != n || (uintptr_t)c % 16 != 0;
+    const size_t b_bytes = copy_b ? align((size_t)k * np) : 0;
+    // per row of a piece: its bytes of A, of a_scale and (when C is staged) of C; a quarter of what is left after B is
+    // kept for the piece's split-K partial sums (launch_locked cuts the split down to what fits)
+    const size_t per_row = (size_t)k + (size_t)qk * sizeof(float) + (copy_c ? (size_t)np * 2 : 0);
+    const size_t left = mem.fixed_left() > b_bytes ? mem.fixed_left() - b_bytes : 0;
+    long rows_fit = (long)((left - left / 4) / per_row) / 16 * 16 - 16;
+    if (b_bytes > mem.fixed_left() / 2 || rows_fit < 16) {
+        hipLaunchKernelGGL(rf::gemm_fp8_blockscale_checked, dim3(ceil_div(n, 16), ceil_div(m, 16)), dim3(64), 0, stream,
+                           (const uint8_t *)a, (const uint8_t *)b, as, bs, (uint16_t *)c, m, m, n, k);
+        RF_HIP(hipGetLastError());
+        return RF_OK;
+    }
+    int rc = RF_OK;
+    const void *b2 = b;
+    if (copy_b) {
+        uint8_t *pb = nullptr;
+        rc = mem.pad(b_bytes, &pb);
+        if (rc != RF_OK) return rc;
+        hipLaunchKernelGGL(pad_group_rows<uint8_t>, pad_grid(np, 1, k), dim3(256), 0, stream, (const uint8_t *)b, n, np, k, 1,
+                           pb, one_group(n, np));
+        RF_HIP(hipGetLastError());
+        b2 = pb;
+    }
+    const size_t base = mem.fixed_used;
+    const int pieces = ceil_div(m, (int)(rows_fit < m ? rows_fit : m));
+    const int rows_per = (ceil_div(m, pieces) + 15) / 16 * 16;           // even pieces, whole m-tiles
+    for (int r0 = 0; r0 < m; r0 += rows_per) {
+        const int rows = m - r0 < rows_per ? m - r0 : rows_per, rp = pad16(rows);
+        mem.fixed_used = base;                                            // the pieces take turns in the same memory
+        uint8_t *pa = nullptr, *psa = nullptr, *pc = nullptr;
+        if ((rc = mem.pad(align((size_t)k * rp), &pa)) != RF_OK) return rc;
+        if ((rc = mem.pad(align((size_t)qk * rp * sizeof(float)), &psa)) != RF_OK) return rc;
+        if (copy_c && (rc = mem.pad(align((size_t)rp * np * 2), &pc)) != RF_OK) return rc;
+        // columns r0 .. r0 + rows - 1 of the caller's [K][m] matrices, padded to rp columns
+        launch_pad_a_and_scales((const uint8_t *)a + r0, as + r0, m, rp, k, 1, pa, (float *)psa, one_group(rows, rp), stream);
+        RF_HIP(hipGetLastError());
+        rf_gemm_config cfg;
+        select_config(rp, np, k, s.num_cu, true, shared().user_plans, &cfg);
+        void *c_piece = copy_c ? (void *)pc : (void *)((uint16_t *)c + (size_t)r0 * n);
+        rc = launch_locked(s, mem, pa, b2, (const float *)psa, bs, c_piece, rp, np, k, &cfg, stream, copy_c ? rp : rows);
+        if (rc != RF_OK) return rc;
+        if (copy_c)
+            RF_HIP(hipMemcpy2DAsync((uint16_t *)c + (size_t)r0 * n, (size_t)n * 2, pc, (size_t)np * 2, (size_t)n * 2, rows,
+                                    hipMemcpyDeviceToDevice, stream));
+    }
+    return RF_OK;
+}
+
 int launch_padded(State &s, Mem &mem, const void *a, const void *b, const float *as, const float *bs, void *c, int m, int n,
                   int k, hipStream_t stream) {
     auto pad16 = [](int x) { return x < 16 ? 16 : (x + 15) / 16 * 16; };
@@ -733,6 +855,7 @@ int launch_padded(State &s, Mem &mem, const void *a, const void *b, const float 
     const size_t off_b = off;  off += copy_b ? align((size_t)k * np) : 0;
     const size_t off_sa = off; off += copy_sa ? align((size_t)qk * mp * sizeof(float)) : 0;
     const size_t off_c = off;  off += copy_c ? align((size_t)mp * np * 2) : 0;
+    if (mem.fixed && off > mem.fixed_left()) return launch_padded_in_pieces(s, mem, a, b, as, bs, c, m, n, k, stream);
     uint8_t *pad = nullptr;
     int rc = mem.pad(off, &pad);
     if (rc != RF_OK) return rc;
@@ -774,12 +897,8 @@ int launch(const void *a, const void *b, const float *as, const float *bs, void 
     int rc = ensure_device_info(s);
     if (rc != RF_OK) return rc;
     Mem mem{s};
-    if (static_memory) {
-        mem.fixed = s.static_scratch;
-    } else {
-        rc = buffers_of(s, stream, &mem.sb);
-        if (rc != RF_OK) return rc;
-    }
+    mem.stream = stream;
+    if (static_memory) mem.fixed = s.static_scratch;
     if (!user_cfg && !tiled_path_ok(a, b, c, m, n) && (double)m * n * k >= kPadThresholdMacs)
         return launch_padded(s, mem, a, b, as, bs, c, m, n, k, stream);
     return launch_locked(s, mem, a, b, as, bs, c, m, n, k, user_cfg, stream);
@@ -877,6 +996,22 @@ int rf_gemm_select_config(int m, int n, int k, rf_gemm_config *out) {
         return RF_OK;
     }
     select_config(m, n, k, s.num_cu, tiled, shared().user_plans, out);
+    return RF_OK;
+}
+
+int rf_gemm_plan_for(int m, int n, int k, int num_cu, rf_gemm_config *out) {
+    g_last_error.clear();
+    if (!out) return fail(RF_ERR_NULL_POINTER, "out is null");
+    if (m < 1 || n < 1 || k < rf::BK || k % rf::BK != 0 || num_cu < 1) return fail(RF_ERR_BAD_SHAPE, "unsupported shape");
+    std::lock_guard<std::mutex> lock(shared().mu);
+    const bool tiled = m >= 16 && n >= 16 && m % 16 == 0 && n % 16 == 0;
+    if (!tiled && (double)m * n * k >= kPadThresholdMacs) {
+        m = m < 16 ? 16 : (m + 15) / 16 * 16;
+        n = n < 16 ? 16 : (n + 15) / 16 * 16;
+        select_config(m, n, k, num_cu, true, shared().user_plans, out);
+        return RF_OK;
+    }
+    select_config(m, n, k, num_cu, tiled, shared().user_plans, out);
     return RF_OK;
 }
 
@@ -1032,10 +1167,6 @@ long grouped_tiles(const GroupedVariant &v, const int *row_offsets, int groups, 
 }
 }  // namespace
 
-extern "C" {
-
-}  // extern "C"
-
 namespace {
 // prepadded: a and as already hold every group from a multiple of 16 rows on (the layout rf_quantize_a_grouped_* writes
 // and rf_grouped_padded_offsets describes); otherwise they hold the groups back to back as row_offsets says.
@@ -1102,10 +1233,8 @@ int grouped_gemm(const void *a, const void *b, const float *as, const float *bs,
         for (int g = 0; g <= rf::kMaxGroups; g++) table.out_row_start[g] = row_offsets[g < groups ? g : groups];
         m_rows = at;
         const size_t a_bytes = ((size_t)k * m_rows + 255) / 256 * 256;
-        StreamBuffers *sb = nullptr;
-        rc = buffers_of(s, stream, &sb);
-        if (rc != RF_OK) return rc;
-        Mem mem{s, sb};
+        Mem mem{s};
+        mem.stream = stream;
         uint8_t *pad = nullptr;
         rc = mem.pad(a_bytes + (size_t)qk * m_rows * sizeof(float), &pad);
         if (rc != RF_OK) return rc;

@@ -44,7 +44,7 @@ EXPORTS = ("run", "rf_fp8_gemm", "rf_fp8_gemm_ex", "rf_gemm_select_config", "rf_
            "rf_gemm_last_error", "rf_fp8_gemm_grouped", "rf_quantize_a_f32", "rf_quantize_a_bf16", "rf_quantize_b_f32", "rf_quantize_b_bf16",
            "rf_cast_f32_to_e4m3fn", "rf_gemm_load_plans", "rf_gemm_clear_plans", "rf_fp8_gemm_time", "rf_fp8_gemm_static",
            "rf_gemm_static_scratch_bytes", "rf_grouped_padded_offsets", "rf_quantize_a_grouped_f32",
-           "rf_quantize_a_grouped_bf16", "rf_fp8_gemm_grouped_padded")
+           "rf_quantize_a_grouped_bf16", "rf_fp8_gemm_grouped_padded", "rf_gemm_plan_for")
 
 
 def lib():
@@ -71,6 +71,8 @@ def lib():
         L.rf_fp8_gemm_time.restype = i32
         L.rf_gemm_select_config.argtypes = [i32, i32, i32, ctypes.POINTER(GemmConfig)]
         L.rf_gemm_select_config.restype = i32
+        L.rf_gemm_plan_for.argtypes = [i32, i32, i32, i32, ctypes.POINTER(GemmConfig)]
+        L.rf_gemm_plan_for.restype = i32
         L.rf_gemm_load_plans.argtypes = [ctypes.c_char_p, ctypes.POINTER(i32)]
         L.rf_gemm_load_plans.restype = i32
         L.rf_gemm_clear_plans.restype = None
@@ -324,6 +326,15 @@ def select_config(m, n, k):
     rc = lib().rf_gemm_select_config(m, n, k, ctypes.byref(cfg))
     if rc != RF_OK:
         raise RuntimeError("rf_gemm_select_config failed (%d): %s" % (rc, last_error()))
+    return cfg
+
+
+def plan_for(m, n, k, num_cu):
+    """The plan for (m, n, k) on a device with num_cu compute units, worked out on the host alone (rf_gemm_plan_for)."""
+    cfg = GemmConfig()
+    rc = lib().rf_gemm_plan_for(m, n, k, num_cu, ctypes.byref(cfg))
+    if rc != RF_OK:
+        raise RuntimeError("rf_gemm_plan_for failed (%d): %s" % (rc, last_error()))
     return cfg
 
 

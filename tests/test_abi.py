@@ -171,3 +171,54 @@ def test_tuner_never_writes_a_stream_k_winner_into_a_table_or_plan_file(tmp_path
     t.emit_plans({(512, 512, 256): [cand(1, 10.0), cand(0, 12.0)], (256, 256, 256): [cand(1, 9.0)]}, str(out))
     lines = [l for l in out.read_text().splitlines() if l.startswith("{")]
     assert len(lines) == 1 and lines[0].startswith("{512, 512, 256, 0, 1, 4, 0}")
+
+
+def test_planner_arithmetic_on_the_host_for_any_compute_unit_count(tmp_path):
+    """rf_gemm_plan_for needs no device. With 256 compute units a tabled shape gets its tabled plan; with any other count
+    the table (measured on 256) is left aside and the cost model counts rounds for the count given: every plan names an
+    existing variant and a split that leaves each part a K block, the persistent schedules only where the shape allows
+    them, the half-tile schedule only when the last round of 256 x 256 tiles on that many units is at most half full,
+    never stream-K, and the skinny-K schedule for one or two K blocks with a large C whatever the count. A loaded plan
+    file still wins on every count."""
+    import radeonflow_kernels_amd as rfk
+    inc = os.path.join(ROOT, "radeonflow_kernels_amd", "csrc", "tuned_plans.inc")
+    table = {p[:3]: p[3:] for p in (tuple(int(x) for x in re.findall(r"-?\d+", l.split("}")[0])) for l in open(inc)
+                                     if l.startswith("{"))}
+    for shape in ((6144, 4608, 7168), (1024, 1536, 7168), (1024, 576, 7168), (6144, 7168, 256)):
+        c = rfk.plan_for(*shape, 256)
+        assert (c.variant, c.split_k, c.group_m, c.stream_k) == table[shape]
+    nv = rfk.lib().rf_gemm_num_variants()
+    for ncu in (8, 64, 104, 128, 228, 304):
+        for (m, n, k) in list(table)[::7] + [(8192, 4608, 7168), (4096, 4096, 4096), (640, 640, 640), (48, 48, 128)]:
+            c = rfk.plan_for(m, n, k, ncu)
+            assert 0 <= c.variant < nv and 1 <= c.split_k <= k // 128 and c.stream_k in (0, 2, 3, 4), (ncu, m, n, k, c)
+            bm, bn = ctypes.c_int(), ctypes.c_int()
+            assert rfk.lib().rf_gemm_variant_info(c.variant, ctypes.byref(bm), ctypes.byref(bn), None, None, None) == 0
+            if c.stream_k in (2, 3):
+                assert c.split_k == 1 and m >= bm.value and n % bn.value == 0 and (k // 128) % 2 == 0
+            if c.stream_k == 3:
+                tiles = -(-m // 256) * (n // 256)
+                left = tiles % ncu
+                assert c.variant == 0 and tiles >= ncu and 0 < left and (left + 7) // 8 * 8 + left <= ncu
+            if c.stream_k == 4:
+                assert k in (128, 256) and m % 16 == 0 and n % 64 == 0
+        assert rfk.plan_for(6144, 7168, 256, ncu).stream_k == 4
+        assert rfk.plan_for(2048, 2048, 256, ncu).stream_k != 4            # below six million outputs
+    # fewer units, more rounds: 2048 x 2048 x 7168 is 64 tiles of 256 x 256: no K split is worth it on 8 units
+    assert rfk.plan_for(2048, 2048, 7168, 8).split_k == 1
+    # ragged shapes are planned at their padded size
+    c, d = rfk.plan_for(1000, 1530, 1024, 128), rfk.plan_for(1008, 1536, 1024, 128)
+    assert (c.variant, c.split_k, c.stream_k) == (d.variant, d.split_k, d.stream_k)
+    plans = tmp_path / "p.plans"
+    plans.write_text("4096 4096 4096 1 2 4 0\n")
+    try:
+        assert rfk.load_plans(str(plans)) == 1
+        for ncu in (64, 256):
+            c = rfk.plan_for(4096, 4096, 4096, ncu)
+            assert (c.variant, c.split_k, c.group_m, c.stream_k) == (1, 2, 4, 0)
+    finally:
+        rfk.clear_plans()
+    cfg = rfk.GemmConfig()
+    assert rfk.lib().rf_gemm_plan_for(16, 16, 100, 256, ctypes.byref(cfg)) == 1
+    assert rfk.lib().rf_gemm_plan_for(16, 16, 128, 0, ctypes.byref(cfg)) == 1
+    assert rfk.lib().rf_gemm_plan_for(16, 16, 128, 256, None) == 2

@@ -76,6 +76,77 @@ def test_run_with_metrics_then_a_call_that_grows_the_buffers_does_not_wait_for_t
     assert np.array_equal(bf16_bits(big[4]), exp_big)
 
 
+def test_more_streams_than_buffer_sets(rfk):
+    """Only launches that need temporary memory take a buffer set, and there are 32 sets per device. 40 streams (made
+    with hipStreamCreate: torch hands out 32 distinct ones) run a one-kernel plan each (no set is used, nothing changes
+    hands), then 32 of them run a split-K plan (all sets taken), then a 33rd does: the least recently used set changes
+    hands without a host wait, and the results stay bit-exact. The same on a stream that is being captured into a graph
+    is refused with RF_ERR_BAD_CONFIG, the capture stays valid, and rf_fp8_gemm_static records the same GEMM into it
+    instead; the replayed graph gives the same bits."""
+    hip = ctypes.CDLL("libamdhip64.so")
+    L = rfk.lib()
+    L.rf_gemm_destroy()
+    direct = exact_problem(256, 256, 256, 31)
+    exp_direct = oracle_bf16(direct)
+    assert rfk.select_config(256, 256, 256).split_k == 1
+    split = exact_problem(128, 512, 7168, 32)
+    exp_split = oracle_bf16(split)
+    assert rfk.select_config(128, 512, 7168).split_k > 1
+    handles = []
+    for _ in range(40):
+        h = ctypes.c_void_p()
+        assert hip.hipStreamCreate(ctypes.byref(h)) == 0
+        handles.append(h)
+    assert len({h.value for h in handles}) == 40
+
+    def launch(fn, g, h):
+        a, b, sa, sb, c = g
+        return fn(a.data_ptr(), b.data_ptr(), sa.data_ptr(), sb.data_ptr(), c.data_ptr(), a.shape[0], b.shape[0],
+                  a.shape[1], h)
+
+    try:
+        gd = [to_gpu(direct) for _ in handles]
+        gs = [to_gpu(split) for _ in range(34)]
+        torch.cuda.synchronize()
+        for g, h in zip(gd, handles):
+            assert launch(L.rf_fp8_gemm, g, h) == 0
+        torch.cuda.synchronize()
+        assert all(np.array_equal(bf16_bits(g[4]), exp_direct) for g in gd)
+        for g, h in zip(gs[:33], handles[:33]):          # the 33rd takes over the first stream's set
+            assert launch(L.rf_fp8_gemm, g, h) == 0
+        gs[0][4].zero_()
+        torch.cuda.synchronize()
+        assert launch(L.rf_fp8_gemm, gs[0], handles[0]) == 0     # and the first stream takes over the second's
+        torch.cuda.synchronize()
+        assert all(np.array_equal(bf16_bits(g[4]), exp_split) for g in gs[:33])
+        # a 34th stream that needs temporary memory, under capture: refused, and the capture goes on
+        cap, g = handles[35], gs[33]
+        graph, graph_exec = ctypes.c_void_p(), ctypes.c_void_p()
+        assert hip.hipStreamBeginCapture(cap, 2) == 0            # hipStreamCaptureModeRelaxed
+        rc = launch(L.rf_fp8_gemm, g, cap)
+        msg = L.rf_gemm_last_error().decode()
+        rc_static = launch(L.rf_fp8_gemm_static, g, cap)
+        assert hip.hipStreamEndCapture(cap, ctypes.byref(graph)) == 0
+        assert rc == 4 and "captured" in msg, (rc, msg)
+        assert rc_static == 0
+        assert hip.hipGraphInstantiate(ctypes.byref(graph_exec), graph, None, None, 0) == 0
+        g[4].zero_()
+        torch.cuda.synchronize()
+        for _ in range(2):
+            assert hip.hipGraphLaunch(graph_exec, cap) == 0
+            assert hip.hipStreamSynchronize(cap) == 0
+            assert np.array_equal(bf16_bits(g[4]), exp_split)
+            g[4].zero_()
+            torch.cuda.synchronize()
+        hip.hipGraphExecDestroy(graph_exec)
+        hip.hipGraphDestroy(graph)
+    finally:
+        torch.cuda.synchronize()
+        L.rf_gemm_destroy()
+        for h in handles:
+            hip.hipStreamDestroy(h)
+
+
 def test_stream_k_plan_for_a_shape_with_fewer_tiles_than_compute_units_is_skipped(rfk, tmp_path):
     """A stream-K plan splits each tile between at most two workgroups, which needs at least one tile per compute unit.
     A plan file that asks for it on a smaller shape is ignored for that shape; the result stays bit-exact."""

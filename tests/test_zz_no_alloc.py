@@ -48,25 +48,47 @@ def test_static_entry_matches_the_allocating_entry_on_two_calls_in_a_row(rfk):
                                "static %r" % (shape,))
 
 
-def test_static_entry_rejects_shapes_beyond_its_scratch_array(rfk):
-    """A ragged M of 6008 with K = 7168 needs a 43 MB staging copy of A: refused with the size in the message, C is
-    not touched, and the entry point keeps working afterwards."""
+def test_static_entry_fits_the_plan_to_its_scratch_array(rfk, tmp_path):
+    """Shapes whose plan under rf_fp8_gemm needs more than the 32 MiB array still run, and allocate nothing:
+    * M = 5001 with K = 7168 (a 36 MB staging copy of A): computed in row ranges that take turns in the array;
+    * the same with a ragged N as well (B and C are staged too);
+    * a plan file that asks for four K parts of 16.8 MB each: cut down to one part;
+    * a stream-K plan from a plan file: replaced by the automatic plan.
+    Exact data, so every fitted plan must give the oracle's bits (and rf_fp8_gemm's); then data with rounding in it
+    against the oracle within tolerance; the canary behind C stays intact; a small split-K shape afterwards still matches
+    rf_fp8_gemm bit for bit (the array holds the earlier calls' data)."""
+    from helpers import exact_problem
     L = rfk.lib()
-    m, n, k = 6008, 512, 7168
-    a = torch.zeros((k, m), dtype=torch.uint8, device="cuda")
-    b = torch.zeros((k, n), dtype=torch.uint8, device="cuda")
-    sa = torch.ones((k // 128, m), dtype=torch.float32, device="cuda")
-    sb = torch.ones((k // 128, n // 128), dtype=torch.float32, device="cuda")
-    c = torch.full((m, n), -5.0, dtype=torch.bfloat16, device="cuda")
-    rc = L.rf_fp8_gemm_static(a.data_ptr(), b.data_ptr(), sa.data_ptr(), sb.data_ptr(), c.data_ptr(), m, n, k, None)
-    torch.cuda.synchronize()
-    assert rc == 4
-    msg = L.rf_gemm_last_error().decode()
-    assert "rf_fp8_gemm_static" in msg and "bytes of scratch memory" in msg and str(32 << 20) in msg
-    assert bool((c == -5.0).all())
-    assert L.rf_fp8_gemm(a.data_ptr(), b.data_ptr(), sa.data_ptr(), sb.data_ptr(), c.data_ptr(), m, n, k, None) == 0
-    torch.cuda.synchronize()
-    assert bool((c == 0).all())
+
+    def static_run(data, canary=4096):
+        g, buf = to_gpu(data, canary_elems=canary)
+        g[4].fill_(-3.0)
+        free_before = torch.cuda.mem_get_info()[0]
+        rfk.fp8_mm_static(*g)
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before, "the call changed the amount of free device memory"
+        assert bool((buf[g[4].numel():].float() == -7.0).all()), "store past the end of C"
+        return g[4]
+
+    for (m, n, k) in ((5001, 512, 7168), (5001, 500, 7168)):
+        assert k * ((m + 15) // 16 * 16) > (32 << 20)
+        data = exact_problem(m, n, k, seed=m + n)
+        assert np.array_equal(bf16_bits(static_run(data)), oracle_bf16(data)), (m, n, k)
+        noisy = rk.generate_input_blockquant(m, n, k, seed=m)
+        assert_close_to_oracle(static_run(noisy), oracle_bf16(noisy), RTOL, ATOL, "static, row ranges %r" % ((m, n, k),))
+    plans = tmp_path / "big.plans"
+    plans.write_text("2048 2048 1024 1 4 8 0\n4096 4096 512 0 1 8 1\n")
+    try:
+        assert rfk.load_plans(str(plans)) == 2
+        for (m, n, k) in ((2048, 2048, 1024), (4096, 4096, 512)):
+            got = rfk.select_config(m, n, k)
+            assert (got.split_k, got.stream_k) == ((4, 0) if k == 1024 else (1, 1))
+            data = exact_problem(m, n, k, seed=k)
+            assert np.array_equal(bf16_bits(static_run(data)), oracle_bf16(data)), (m, n, k)
+            noisy = rk.generate_input_blockquant(m, n, k, seed=k + 1)
+            assert_close_to_oracle(static_run(noisy), oracle_bf16(noisy), RTOL, ATOL, "static, fitted plan %r" % ((m, n, k),))
+    finally:
+        rfk.clear_plans()
     data = rk.generate_input_blockquant(256, 1536, 7168, 25)
     got, want = _both(rfk, data)
     assert np.array_equal(got, want)
