@@ -61,7 +61,8 @@ def kernel_source_sha():
 
 
 def measured_traffic(config, cfg):
-    """HBM-side bytes per launch from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summaries under profiles/ (lines
+    """HBM-side bytes per GEMM, summed over every kernel the plan launches (a split-K plan: the partial-sum kernel and
+    the reduction), from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summaries under profiles/ (lines
     '@traffic config=C2 plan=0,1,2 fetch_kib=... write_kib=... fetch_factor=... write_factor=... source_sha=...').
     Returns (bytes, note), or (None, why) when there is no summary for this configuration and plan or when the kernel
     sources have changed since it was taken."""
@@ -83,7 +84,7 @@ def measured_traffic(config, cfg):
                 continue
             fetch = float(kv["fetch_kib"]) * float(kv["fetch_factor"]) * 1024
             write = float(kv["write_kib"]) * float(kv["write_factor"]) * 1024
-            return fetch + write, "fetch %.1f MB + write %.1f MB per launch, profiles/%s" % (
+            return fetch + write, "fetch %.1f MB + write %.1f MB per GEMM (all its kernels), profiles/%s" % (
                 fetch / 1e6, write / 1e6, os.path.basename(path))
     return None, why
 
@@ -131,6 +132,28 @@ def time_gemm(rfk, sets, steps, warmup, stream):
         stream.synchronize()
         torch.cuda.synchronize()
     return e0.elapsed_time(e1) * 1e3 / steps
+
+
+def cold_operands_us(rfk, g, m, n, k, steps, warmup, stream):
+    """Microseconds per GEMM with operands that are not in the 256 MB Infinity Cache: enough copies of the operand set
+    in rotation that a set is evicted before its turn comes again. Returns (us, copies, bytes of all copies)."""
+    set_bytes = algorithmic_bytes(m, n, k)
+    ncopies = max(3, int(2 * 256e6 / set_bytes) + 1)
+    sets = [g] + [tuple(t.clone() for t in g) for _ in range(ncopies - 1)]
+    us = time_gemm(rfk, sets, max(steps, 2 * ncopies), max(warmup, 2 * ncopies), stream)
+    del sets
+    return us, ncopies, ncopies * set_bytes
+
+
+def roofline_of_work(flop, nbytes, us):
+    """The same for any launch given its algorithmic FLOP and bytes (the grouped form: every expert's weights, every
+    row of A and of C once)."""
+    tflops, gbs = flop / us / 1e6, nbytes / us / 1e3
+    if flop / (PEAK_FP8_TFLOPS * 1e12) >= nbytes / (PEAK_HBM_GBS * 1e9):
+        return {"bound": "mfma", "achieved": round(tflops, 2), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(tflops / PEAK_FP8_TFLOPS, 4), "algorithmic_flop": flop, "algorithmic_bytes": nbytes}
+    return {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "frac": round(gbs / PEAK_HBM_GBS, 4), "algorithmic_flop": flop, "algorithmic_bytes": nbytes}
 
 
 def roofline_of(m, n, k, us):
@@ -233,7 +256,7 @@ def parity_report(rfk, cref, rk, data, g, stream, expect=None, truth_rows=64):
             "elements": int(m * n), "pass": bad == 0}
 
 
-def measure_config(rfk, cref, rk, name, steps, warmup, stream, with_cpu, settle_seconds, keep=False):
+def measure_config(rfk, cref, rk, name, steps, warmup, stream, with_cpu, settle_seconds, keep=False, cold_too=True):
     """One configuration: inputs, settled launch time, roofline fraction, correctness gate. Returns the record (and
     the inputs with keep=True)."""
     m, n, k, seed = {**CONFIGS, **EXTRA_CONFIGS}[name]
@@ -257,6 +280,11 @@ def measure_config(rfk, cref, rk, name, steps, warmup, stream, with_cpu, settle_
     traffic, note = measured_traffic(name, cfg)
     rec["roofline"]["traffic"] = traffic
     rec["roofline"]["traffic_note"] = note
+    if cold_too:
+        us_cold, ncopies, nbytes = cold_operands_us(rfk, g, m, n, k, max(steps, 50), max(warmup, 50), stream)
+        rec["cold_operands"] = {"us_per_gemm": round(us_cold, 2), "frac": roofline_of(m, n, k, us_cold)["frac"],
+                                "note": "%d operand sets in rotation (%.0f MB > 256 MB Infinity Cache), launches from Python"
+                                        % (ncopies, nbytes / 1e6)}
     expect = cpu_s = None
     if with_cpu:
         a, b, sa, sb, c = data
@@ -289,6 +317,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity gate")
     ap.add_argument("--settle", type=float, default=SETTLE_SECONDS, help="seconds of launches before the timed region")
     ap.add_argument("--no-clock", action="store_true", help="skip the 0.6 s clock and power read-out (shorter profiler traces)")
+    ap.add_argument("--timed-only", action="store_true",
+                    help="with --config: stop after the settled, timed launches (for profiler runs: the last --steps "
+                         "launches of the trace are then exactly the timed region)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (output tiles are independent: "
@@ -309,20 +340,31 @@ def main():
 
     headline = args.config or "C2"
     m, n, k, seed = {**CONFIGS, **EXTRA_CONFIGS}[headline]
+    if args.timed_only:
+        if not args.config:
+            print("bench.py: --timed-only needs --config", file=sys.stderr)
+            return 2
+        mm, nn, kk, seed_ = {**CONFIGS, **EXTRA_CONFIGS}[args.config]
+        gg = to_gpu(rk.generate_input_blockquant(mm, nn, kk, seed_))
+        us_, settle_ = settled_us(rfk, gg, args.steps, args.warmup, args.settle)
+        cfg_ = rfk.select_config(mm, nn, kk)
+        print(json.dumps({"config": args.config, "us_per_gemm": round(us_, 2), "steps": args.steps, "warmup": args.warmup,
+                          "settle_launches": settle_, "roofline": roofline_of(mm, nn, kk, us_),
+                          "plan": {"variant": cfg_.variant, "split_k": cfg_.split_k, "group_m": cfg_.group_m,
+                                   "stream_k": cfg_.stream_k}}))
+        return 0
     rec, data, g, gen_s, us_burst, cpu_s = measure_config(rfk, cref, rk, headline, args.steps, args.warmup, stream,
-                                                          not args.no_cpu, args.settle, keep=True)
+                                                          not args.no_cpu, args.settle, keep=True, cold_too=False)
     us = rec["us_per_gemm"]
     flop = 2.0 * m * n * k
     tflops = flop / us / 1e6
     with torch.cuda.stream(stream):
         rfk.fp8_mm_time(*g, warmup=rec["settle_launches"] // 2, iters=1)      # the clock falls back within milliseconds
     samples = sorted(per_launch_us(rfk, g, max(20, min(args.steps, 200)), stream))
-    # operands that are not in the 256 MB Infinity Cache: rotate enough copies that a set is evicted before its turn
-    set_bytes = algorithmic_bytes(m, n, k)
-    ncopies = max(3, int(2 * 256e6 / set_bytes) + 1)
-    cold_sets = [g] + [tuple(t.clone() for t in g) for _ in range(ncopies - 1)]
-    us_cold = time_gemm(rfk, cold_sets, max(args.steps, 50), max(args.warmup, 50), stream)
-    del cold_sets
+    us_cold, ncopies, cold_bytes = cold_operands_us(rfk, g, m, n, k, max(args.steps, 50), max(args.warmup, 50), stream)
+    rec["cold_operands"] = {"us_per_gemm": round(us_cold, 2), "frac": roofline_of(m, n, k, us_cold)["frac"],
+                            "note": "%d operand sets in rotation (%.0f MB > 256 MB Infinity Cache), launches from Python"
+                                    % (ncopies, cold_bytes / 1e6)}
     roofline = dict(rec["roofline"])
     roofline["kernel"] = rec["kernel"]
     roofline["avg_launch_us"] = round(us, 2)
@@ -339,8 +381,9 @@ def main():
                              "note": "the first %d launches of the process after %d warm-up launches: shader clock and "
                                      "board power have not reached their state under load" % (args.steps, args.warmup)},
         "cold_operands": {"us_per_gemm": round(us_cold, 2), "tflops": round(flop / us_cold / 1e6, 2),
+                          "pct_fp8_mfma_peak": round(100 * flop / us_cold / 1e6 / PEAK_FP8_TFLOPS, 2),
                           "note": "%d operand sets in rotation (%.0f MB > 256 MB Infinity Cache)"
-                                  % (ncopies, ncopies * set_bytes / 1e6)},
+                                  % (ncopies, cold_bytes / 1e6)},
         "pct_fp8_mfma_peak": round(100 * tflops / PEAK_FP8_TFLOPS, 2),
         "achieved_hbm_gbs_algorithmic": rec["gbs_algorithmic"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3fn",
@@ -367,8 +410,8 @@ def main():
 
     if args.config is None:
         # all five configurations: settled time, roofline fraction and the same correctness gate
-        print("%-3s %-16s %9s %9s %6s %6s %9s %9s  %s" % ("cfg", "shape", "us", "TFLOP/s", "bound", "frac", "bad@1e-2",
-              "bad@1e-3", "plan"), file=sys.stderr)
+        print("%-3s %-16s %9s %9s %9s %6s %6s %9s %9s  %s" % ("cfg", "shape", "us", "us cold", "TFLOP/s", "bound", "frac",
+              "bad@1e-2", "bad@1e-3", "plan"), file=sys.stderr)
         out["all_configs"] = {}
         for name in sorted(CONFIGS):
             if name == headline:
@@ -381,8 +424,9 @@ def main():
                                    min(args.settle, 0.25))
             out["all_configs"][name] = r
             par = r.get("parity")
-            print("%-3s %-16s %9.2f %9.1f %6s %6.3f %9s %9s  %r" % (
-                name, "%dx%dx%d" % tuple(r["shape"]), r["us_per_gemm"], r["tflops"], r["roofline"]["bound"],
+            print("%-3s %-16s %9.2f %9.2f %9.1f %6s %6.3f %9s %9s  %r" % (
+                name, "%dx%dx%d" % tuple(r["shape"]), r["us_per_gemm"], r["cold_operands"]["us_per_gemm"], r["tflops"],
+                r["roofline"]["bound"],
                 r["roofline"]["frac"], par["mismatches"] if par else "-",
                 par["mismatches_at_reference_atol_1e-3"] if par else "-", r["plan"]), file=sys.stderr)
 
@@ -450,7 +494,8 @@ def main():
                             gm_, min(sizes), max(sizes), gn, gk),
                         "us": round(u, 2), "tflops": round(tf, 1), "pct_fp8_mfma_peak": round(100 * tf / PEAK_FP8_TFLOPS, 2),
                         "algorithmic_mb": round(gbytes / 1e6, 1), "gbs": round(gbytes / u / 1e3, 1),
-                        "pct_hbm_peak": round(100 * gbytes / u / 1e3 / PEAK_HBM_GBS, 2)}
+                        "pct_hbm_peak": round(100 * gbytes / u / 1e3 / PEAK_HBM_GBS, 2),
+                        "roofline": roofline_of_work(2.0 * gm_ * gn * gk, gbytes, u)}
             print("%s %s: %.2f us  %.1f TFLOP/s (%.1f %% of the fp8 peak), %.0f GB/s algorithmic (%.1f %% of 8 TB/s)" % (
                   key, out[key]["workload"], u, tf, 100 * tf / PEAK_FP8_TFLOPS, gbytes / u / 1e3,
                   100 * gbytes / u / 1e3 / PEAK_HBM_GBS), file=sys.stderr)
@@ -478,7 +523,9 @@ def main():
         out["grouped_any_sizes_padded_layout"] = {
             "workload": out["grouped_any_sizes"]["workload"] + ", activations written by quantize_a_grouped",
             "us": round(u, 2), "tflops": round(tf, 1), "pct_fp8_mfma_peak": round(100 * tf / PEAK_FP8_TFLOPS, 2),
-            "quantize_a_grouped_bf16_us": round(uq, 2)}
+            "quantize_a_grouped_bf16_us": round(uq, 2),
+            "roofline": roofline_of_work(2.0 * gm_any * gn * gk,
+                                         gm_any * gk + gg * gn * gk + 2 * gm_any * gn + 4 * (gk // 128) * (gm_any + gg * (gn // 128)), u)}
         print("grouped_any_sizes_padded_layout: %.2f us  %.1f TFLOP/s (quantize_a_grouped bf16 -> padded layout: %.2f us, "
               "includes the allocation of its outputs by torch)" % (u, tf, uq), file=sys.stderr)
         del xg, a_pad, sa_pad, ga_any, gsa_any, gc_any
