@@ -151,6 +151,11 @@ int rf_gemm_variant_info(int variant, int *block_m, int *block_n, int *waves_m, 
  * (or if the index is out of range). */
 int rf_gemm_variant_has_stream_k(int variant);
 int rf_gemm_variant_has_persistent(int variant);
+/* Number of wave groups of one workgroup that split K between them (0 if the index is out of range). 1 for the ordinary
+ * variants. A variant with more computes a tile's K parts side by side in one workgroup and sums them through LDS in part
+ * order (the bits of split_k = that many equal parts, in one launch, no partial sums in memory): it takes split_k == 1 and
+ * the tile schedule only, and K/128 must be a multiple of the count (RF_ERR_BAD_CONFIG otherwise). */
+int rf_gemm_variant_k_groups(int variant);
 
 /* Device workspace (split-K partial sums) needed for a shape under the automatic plan, in bytes. The staging copies
  * of ragged or unaligned operands are not part of it: that buffer grows on the first such call. */

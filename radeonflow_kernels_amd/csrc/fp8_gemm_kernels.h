@@ -154,7 +154,9 @@ __device__ __forceinline__ void tile_mainloop(
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // (a workgroup may hold several wave groups of NW waves, each running this loop on its own tile of LDS: the wave's
+    // index inside its group)
+    const int wave = __builtin_amdgcn_readfirstlane((tid >> 6) % NW);
     const int L = lane & 15, g = lane >> 4;
     const int wm = wave % WAVES_M, wn = wave / WAVES_M;
 
@@ -747,6 +749,69 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_til
                                                         M - m0, N - n0, lds);
     else
         store_tile_bf16<BM, BN, WAVES_M, WAVES_N>(acc, (uint16_t *)Cout, M_store, N, m0, n0, lds);
+}
+
+// ---------------------------------------------------------------------------------------------
+// K split inside one workgroup. GROUPS wave groups (NW waves each) compute the same BM x BN tile, group g over K blocks
+// [g * QK / GROUPS, (g + 1) * QK / GROUPS) with LDS stages of its own; then groups 1.. hand their fp32 accumulators to
+// group 0 through LDS, which adds them in group order and stores bf16: the bits of the two-launch form with GROUPS equal
+// K parts (PARTIAL kernel + reduce_splitk_bf16), without the partial sums' trip through memory and without the second
+// launch. Every wave of the workgroup runs the same number of loop iterations (each holds a workgroup-wide barrier), so
+// the host launches it only when QK % GROUPS == 0; the kernel returns at once otherwise.
+// Same argument list as gemm_fp8_blockscale_tile (kb_per_split is not used).
+// ---------------------------------------------------------------------------------------------
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, int GROUPS>
+struct InWgSplitGeom {
+    using G = TileGeom<BM, BN, WAVES_M, WAVES_N, NS>;
+    static constexpr int GROUP_LDS = (G::LDS_BYTES + 1023) / 1024 * 1024;
+    static constexpr int LDS_BYTES = GROUPS * GROUP_LDS;
+    static_assert(LDS_BYTES <= 160 * 1024, "every group's stages fit the CU's LDS");
+    static_assert(G::TM * G::TN * G::NT * 16 <= GROUP_LDS, "a group's accumulators fit its own LDS region");
+    static_assert(G::NT * GROUPS <= 1024, "one workgroup");
+};
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, int GROUPS>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64 * GROUPS) void gemm_fp8_blockscale_tile_ksplit_in_wg(
+    const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
+    const float *__restrict__ SB, void *__restrict__ Cout, int M, int N, int K, int kb_per_split,
+    int tiles_m, int tiles_n, int group_m, int M_store) {
+    using G = TileGeom<BM, BN, WAVES_M, WAVES_N, NS>;
+    using W = InWgSplitGeom<BM, BN, WAVES_M, WAVES_N, NS, GROUPS>;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    const int QK = K / BK;
+    if (QK % GROUPS != 0) return;                           // never launched so: unequal K parts would not meet at the barriers
+    int tile_m, tile_n;
+    tile_of_block(blockIdx.x, tiles_m * tiles_n, tiles_m, tiles_n, group_m, true, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int grp = __builtin_amdgcn_readfirstlane((int)threadIdx.x / G::NT), len = QK / GROUPS;
+    uint8_t *my_lds = lds + grp * W::GROUP_LDS;
+    f32x4 acc[G::TM][G::TN];
+    tile_mainloop<BM, BN, WAVES_M, WAVES_N, NS>(A, B, SA, SB, M, M, N, m0, n0, grp * len, (grp + 1) * len, my_lds, acc);
+    __syncthreads();                                        // every group is done with its stages
+    // accumulators in register order: tile (j, i) of thread t of the group at ((j * TN + i) * NT + t) * 16 bytes
+    f32x4 *mine = (f32x4 *)my_lds + (int)threadIdx.x % G::NT;
+    if (grp > 0) {
+#pragma unroll
+        for (int j = 0; j < G::TM; j++)
+#pragma unroll
+            for (int i = 0; i < G::TN; i++) mine[(j * G::TN + i) * G::NT] = acc[j][i];
+    }
+    __syncthreads();
+    if (grp == 0) {
+#pragma unroll
+        for (int q = 1; q < GROUPS; q++) {
+            const f32x4 *theirs = (const f32x4 *)(lds + q * W::GROUP_LDS) + (int)threadIdx.x % G::NT;
+#pragma unroll
+            for (int j = 0; j < G::TM; j++)
+#pragma unroll
+                for (int i = 0; i < G::TN; i++) {
+                    const f32x4 v = theirs[(j * G::TN + i) * G::NT];
+                    acc[j][i][0] += v[0]; acc[j][i][1] += v[1]; acc[j][i][2] += v[2]; acc[j][i][3] += v[3];
+                }
+        }
+        // staging in group 0's own region, which nobody else touches any more: no barrier (the other groups are gone)
+        store_tile_bf16<BM, BN, WAVES_M, WAVES_N, default_store_passes<BM, WAVES_M>(), false>(acc, (uint16_t *)Cout, M_store, N,
+                                                                                              m0, n0, lds);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -56,8 +56,9 @@ struct Variant {
     persistent_kernel_t persistent;      // null: no persistent form
     int lds_persistent;
     persistent_kernel_t persistent_half_tail = nullptr;   // null: no form that ends with half tiles
+    int k_groups = 1;                    // > 1: wave groups of one workgroup split K between them (needs K/128 % k_groups == 0)
     int lds_bytes() const { return lds; }
-    int threads() const { return waves_m * waves_n * 64; }
+    int threads() const { return waves_m * waves_n * 64 * k_groups; }
 };
 #define RF_VARIANT(BM, BN, WM, WN)                                                         \
     Variant { BM, BN, WM, WN, rf::TileGeom<BM, BN, WM, WN>::LDS_BYTES,                     \
@@ -96,6 +97,10 @@ const Variant kVariants[] = {
     RF_VARIANT_TILE_ONLY_NS3(64, 128, 2, 2),    // 9: variant 7 with three stages, 74 KiB LDS (2 workgroups per CU)
     RF_VARIANT_TILE_ONLY_NS3(128, 256, 2, 4),   // 10: variant 3 with three stages, 149 KiB LDS
     RF_VARIANT_TILE_ONLY_NS3(192, 192, 2, 4),   // 11: variant 5 with three stages, 147 KiB LDS
+    // 12: the 64 x 128 three-stage tile with K split between two wave groups of one workgroup (8 waves, 150 KiB LDS):
+    // the split-K plan of a short, wide-K shape in one launch, with no partial sums in memory
+    Variant{64, 128, 2, 2, rf::InWgSplitGeom<64, 128, 2, 2, 3, 2>::LDS_BYTES,
+            rf::gemm_fp8_blockscale_tile_ksplit_in_wg<64, 128, 2, 2, 3, 2>, nullptr, nullptr, nullptr, 0, nullptr, 2},
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
@@ -202,7 +207,8 @@ int ensure_device_info(State &s) {
     s.num_cu = prop.multiProcessorCount;
     for (const Variant &v : kVariants) {
         RF_HIP(hipFuncSetAttribute((const void *)v.direct, hipFuncAttributeMaxDynamicSharedMemorySize, v.lds_bytes()));
-        RF_HIP(hipFuncSetAttribute((const void *)v.partial, hipFuncAttributeMaxDynamicSharedMemorySize, v.lds_bytes()));
+        if (v.partial)
+            RF_HIP(hipFuncSetAttribute((const void *)v.partial, hipFuncAttributeMaxDynamicSharedMemorySize, v.lds_bytes()));
         if (v.streamk)
             RF_HIP(hipFuncSetAttribute((const void *)v.streamk, hipFuncAttributeMaxDynamicSharedMemorySize, v.lds_bytes()));
         if (v.persistent)
@@ -432,6 +438,7 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
     }
     auto usable = [&](const TunedPlan &p) {
         return p.m == m && p.n == n && p.k == k && p.variant < kNumVariants && p.split_k <= k / rf::BK &&
+               (kVariants[p.variant].k_groups == 1 || (p.split_k == 1 && (k / rf::BK) % kVariants[p.variant].k_groups == 0)) &&
                (p.stream_k != RF_SCHEDULE_PERSISTENT || persistent_ok(kVariants[p.variant], m, n, k)) &&
                (p.stream_k != RF_SCHEDULE_STREAM_K || stream_k_ok(kVariants[p.variant], m, n, num_cu)) &&
                (p.stream_k != RF_SCHEDULE_PERSISTENT_HALF_TAIL || half_tail_ok(kVariants[p.variant], m, n, k, num_cu)) &&
@@ -528,6 +535,10 @@ int launch_locked(State &s, Mem &mem, const void *a, const void *b, const float 
             cfg.split_k > k / rf::BK || (cfg.variant >= 0 && !tiled_ok) || (cfg.variant < 0 && cfg.split_k != 1) ||
             (cfg.stream_k != 0 && (cfg.variant < 0 || cfg.split_k != 1)))
             return fail(RF_ERR_BAD_CONFIG, "configuration not usable for this shape");
+        if (cfg.variant >= 0 && kVariants[cfg.variant].k_groups > 1 &&
+            (cfg.split_k != 1 || cfg.stream_k != RF_SCHEDULE_TILES || (k / rf::BK) % kVariants[cfg.variant].k_groups != 0))
+            return fail(RF_ERR_BAD_CONFIG, "this variant splits K inside the workgroup: it needs split_k == 1, the tile "
+                                           "schedule and a number of K blocks that its wave groups divide");
         if (cfg.stream_k == RF_SCHEDULE_STREAM_K) {
             const Variant &sv = kVariants[cfg.variant];
             if (!sv.streamk) return fail(RF_ERR_BAD_CONFIG, "this variant has no stream_k form");
@@ -1042,6 +1053,10 @@ int rf_gemm_variant_info(int variant, int *block_m, int *block_n, int *waves_m, 
     if (waves_n) *waves_n = v.waves_n;
     if (lds_bytes) *lds_bytes = v.lds_bytes();
     return RF_OK;
+}
+
+int rf_gemm_variant_k_groups(int variant) {
+    return variant >= 0 && variant < kNumVariants ? kVariants[variant].k_groups : 0;
 }
 
 int rf_gemm_variant_has_persistent(int variant) {

@@ -44,7 +44,7 @@ EXPORTS = ("run", "rf_fp8_gemm", "rf_fp8_gemm_ex", "rf_gemm_select_config", "rf_
            "rf_gemm_last_error", "rf_fp8_gemm_grouped", "rf_quantize_a_f32", "rf_quantize_a_bf16", "rf_quantize_b_f32", "rf_quantize_b_bf16",
            "rf_cast_f32_to_e4m3fn", "rf_gemm_load_plans", "rf_gemm_clear_plans", "rf_fp8_gemm_time", "rf_fp8_gemm_static",
            "rf_gemm_static_scratch_bytes", "rf_grouped_padded_offsets", "rf_quantize_a_grouped_f32",
-           "rf_quantize_a_grouped_bf16", "rf_fp8_gemm_grouped_padded", "rf_gemm_plan_for")
+           "rf_quantize_a_grouped_bf16", "rf_fp8_gemm_grouped_padded", "rf_gemm_plan_for", "rf_gemm_variant_k_groups")
 
 
 def lib():
@@ -81,6 +81,8 @@ def lib():
         L.rf_gemm_variant_info.restype = i32
         L.rf_gemm_variant_has_stream_k.argtypes = [i32]
         L.rf_gemm_variant_has_stream_k.restype = i32
+        L.rf_gemm_variant_k_groups.argtypes = [i32]
+        L.rf_gemm_variant_k_groups.restype = i32
         L.rf_gemm_variant_has_persistent.argtypes = [i32]
         L.rf_gemm_variant_has_persistent.restype = i32
         L.rf_gemm_workspace_bytes.argtypes = [i32, i32, i32]
@@ -352,6 +354,14 @@ def clear_plans():
     lib().rf_gemm_clear_plans()
 
 
+def plan_can_run(v, split, k):
+    """Whether variant v (an entry of variants()) takes `split` K parts at this K under the tile schedule: a variant that
+    splits K between wave groups of one workgroup takes split 1 only, and K/128 must be a multiple of its group count."""
+    if split > k // 128:
+        return False
+    return v["k_groups"] == 1 or (split == 1 and (k // 128) % v["k_groups"] == 0)
+
+
 def variants():
     L = lib()
     out = []
@@ -361,5 +371,6 @@ def variants():
         out.append(dict(variant=v, block_m=vals[0].value, block_n=vals[1].value, waves_m=vals[2].value,
                         waves_n=vals[3].value, lds_bytes=vals[4].value,
                         stream_k=bool(L.rf_gemm_variant_has_stream_k(v)),
-                        persistent=bool(L.rf_gemm_variant_has_persistent(v))))
+                        persistent=bool(L.rf_gemm_variant_has_persistent(v)),
+                        k_groups=L.rf_gemm_variant_k_groups(v)))
     return out

@@ -82,6 +82,8 @@ def tune_shape(rfk, m, n, k, log=print):
         for split, sk in [(sp, 0) for sp in SPLITS] + [(1, 1), (1, 2), (1, 3), (1, 4)]:
             if split > k // 128 or (sk == 1 and (tiles < ncu or not v["stream_k"])):
                 continue
+            if sk == 0 and not rfk.plan_can_run(v, split, k):
+                continue
             if sk in (2, 3) and (not v["persistent"] or m < v["block_m"] or m % 16 or n % v["block_n"] or (k // 128) % 2):
                 continue
             if sk == 4 and (v["variant"] != 0 or k > 256 or m % 16 or n % 64):

@@ -58,7 +58,7 @@ def test_every_variant_and_split(rfk, gen, m, n, k):
     exp = oracle_bf16(data)
     for v in rfk.variants():
         for split in (1, 2, 3):
-            if split > k // 128:
+            if not rfk.plan_can_run(v, split, k):
                 continue
             cfg = rfk.GemmConfig(v["variant"], split, 4, 0)
             out = _run(rfk, data, config=cfg, canary=1024)
@@ -78,6 +78,8 @@ def test_split_k_grid_reaches_every_tile_and_split_once(rfk, m, n):
     other = to_gpu(exact_problem(m, n, k, seed=m + n + 1))
     for v in rfk.variants():
         for split in (2, 3, 4, 5, 8, 16):
+            if not rfk.plan_can_run(v, split, k):
+                continue
             cfg = rfk.GemmConfig(v["variant"], split, 3, 0)
             rfk.fp8_mm(*other, config=cfg)                  # fills the workspace with another problem's sums
             out = _run(rfk, data, config=cfg, canary=1024)
@@ -98,7 +100,7 @@ def test_bit_exact_on_exactly_representable_data(rfk, m, n, k):
     plans = [None]
     if tiled:
         plans += [rfk.GemmConfig(v["variant"], s, gm, 0) for v in rfk.variants() for s, gm in ((1, 1), (2, 8), (3, 3))
-                  if s <= k // 128]
+                  if rfk.plan_can_run(v, s, k)]
     for cfg in plans:
         out = _run(rfk, data, config=cfg, canary=1024)
         assert np.array_equal(bf16_bits(out), exp), "plan %r" % (cfg,)
@@ -275,6 +277,40 @@ def test_skinny_k_schedule_bit_exact(rfk, m, n, k):
     out = _run(rfk, noisy, config=cfg, canary=1024)
     assert np.array_equal(bf16_bits(out), ref)
     assert_close_to_oracle(out, oracle_bf16(noisy), RTOL, ATOL, "skinny K")
+
+
+@pytest.mark.parametrize("m,n,k", [(64, 128, 256), (1024, 1536, 7168), (208, 576, 1024), (64, 1536, 7168), (1024, 512, 512)])
+def test_k_split_inside_the_workgroup_equals_the_two_launch_form(rfk, m, n, k):
+    """Variants whose wave groups split K inside one workgroup (partial sums added through LDS in part order) against
+    the same tile with split_k = the number of groups (fp32 partial sums through memory + the reduction kernel): the
+    same bits on data with rounding in it, the oracle's bits on exact data, twice on the same buffers, canary intact;
+    and K block counts their groups do not divide are refused."""
+    tried = 0
+    for v in rfk.variants():
+        if v["k_groups"] < 2:
+            continue
+        twin = [w for w in rfk.variants() if w["k_groups"] == 1 and (w["block_m"], w["block_n"], w["waves_m"], w["waves_n"])
+                == (v["block_m"], v["block_n"], v["waves_m"], v["waves_n"]) and w["lds_bytes"] * v["k_groups"] <= v["lds_bytes"]
+                and w["lds_bytes"] * v["k_groups"] > v["lds_bytes"] - 4096]
+        assert len(twin) == 1, "the one-group variant with the same tile and stage count"
+        cfg, cfg2 = rfk.GemmConfig(v["variant"], 1, 8, 0), rfk.GemmConfig(twin[0]["variant"], v["k_groups"], 8, 0)
+        assert (k // 128) % v["k_groups"] == 0
+        data = exact_problem(m, n, k, seed=m + n + k)
+        exp = oracle_bf16(data)
+        for rep in range(2):
+            assert np.array_equal(bf16_bits(_run(rfk, data, config=cfg, canary=1024)), exp), "rep %d" % rep
+        noisy = rk.generate_input_blockquant(m, n, k, seed=m + k)
+        ref = bf16_bits(_run(rfk, noisy, config=cfg2)).copy()
+        out = _run(rfk, noisy, config=cfg, canary=1024)
+        assert np.array_equal(bf16_bits(out), ref)
+        assert_close_to_oracle(out, oracle_bf16(noisy), RTOL, ATOL, "K split inside the workgroup")
+        for bad in (rfk.GemmConfig(v["variant"], 2, 8, 0), rfk.GemmConfig(v["variant"], 1, 8, 2)):
+            with pytest.raises(RuntimeError):
+                _run(rfk, data, config=bad)
+        with pytest.raises(RuntimeError):                       # three K blocks, two groups
+            _run(rfk, exact_problem(64, 128, 384, seed=1), config=cfg)
+        tried += 1
+    assert tried > 0
 
 
 def test_skinny_k_schedule_rejects_shapes_it_does_not_fit(rfk):
@@ -634,7 +670,7 @@ def test_signed_zeros_and_negative_scales(rfk, m, n, k):
     exp = oracle_bf16(data)
     plans = [None]
     if m % 16 == 0 and n % 16 == 0:
-        plans += [rfk.GemmConfig(v["variant"], s, 4, 0) for v in rfk.variants() for s in (1, 2, 4) if s <= k // 128]
+        plans += [rfk.GemmConfig(v["variant"], s, 4, 0) for v in rfk.variants() for s in (1, 2, 4) if rfk.plan_can_run(v, s, k)]
         plans += [rfk.GemmConfig(v["variant"], 1, 4, 2) for v in rfk.variants()
                   if v["persistent"] and m % v["block_m"] == 0 and n % v["block_n"] == 0 and (k // 128) % 2 == 0]
     for cfg in plans:
@@ -658,7 +694,7 @@ def test_nan_codes_poison_their_row_or_column_only(rfk, m, n, k):
     assert exp_nan[5].all() and exp_nan[m - 1].all() and exp_nan[:, 3].all() and exp_nan.sum() == 2 * n + m - 2
     plans = [None]
     if m % 16 == 0 and n % 16 == 0:
-        plans += [rfk.GemmConfig(v["variant"], s, 4, 0) for v in rfk.variants() for s in (1, 3) if s <= k // 128]
+        plans += [rfk.GemmConfig(v["variant"], s, 4, 0) for v in rfk.variants() for s in (1, 3) if rfk.plan_can_run(v, s, k)]
         plans += [rfk.GemmConfig(v["variant"], 1, 4, 2) for v in rfk.variants()
                   if v["persistent"] and m % v["block_m"] == 0 and n % v["block_n"] == 0 and (k // 128) % 2 == 0]
     for cfg in plans:
