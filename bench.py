@@ -477,7 +477,7 @@ def main():
                                  ("grouped_any_sizes", offs_any, (ga_any, gb, gsa_any, gsb, gc_any))):
             gm_ = offs_[-1]
             with torch.cuda.stream(stream):
-                for _ in range(args.warmup // 4 + 5):
+                for _ in range(max(args.warmup // 4 + 5, 600)):       # ~0.2 s of the same launch: the clock has settled
                     rfk.fp8_mm_grouped(*ops_, offs_)
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record(stream)
@@ -504,7 +504,7 @@ def main():
         xg = torch.randn((gm_any, gk), device="cuda", dtype=torch.bfloat16)
         with torch.cuda.stream(stream):
             a_pad, sa_pad = rfk.quantize_a_grouped(xg, offs_any)
-            for _ in range(args.warmup // 4 + 5):
+            for _ in range(max(args.warmup // 4 + 5, 600)):
                 rfk.fp8_mm_grouped_padded(a_pad, gb, sa_pad, gsb, gc_any, offs_any)
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record(stream)

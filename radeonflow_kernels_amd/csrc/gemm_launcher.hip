@@ -483,8 +483,10 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
     // no padded columns, e.g. N = 576, 1536 or 3072; the 64x128 tile where M is short or the whole problem is a few
     // microseconds); the others never won by more than a few percent.
     struct Candidate { int variant; double c, f; };
+    // (variant 12 splits K between two wave groups of one workgroup: half the K blocks per group, one launch, no reduction
+    // term; fitted on its 103 tabled measurements: the best plan of short shapes, M <= 512, with K = 512 ... 2304)
     const Candidate cands[] = {{0, 0.955, 7.96}, {3, 0.619, 5.11}, {5, 0.71, 5.2},  {6, 0.74, 3.7},  {7, 0.82, 0.0},
-                               {8, 0.52, 4.5},   {9, 0.70, 0.5},   {10, 0.53, 5.9}, {11, 0.62, 5.8}};
+                               {8, 0.52, 4.5},   {9, 0.70, 0.5},   {10, 0.53, 5.9}, {11, 0.62, 5.8}, {12, 0.75, 2.9}};
     const double f_next = 3.0, reduce_fixed = 2.83, reduce_per_elem = 1.37e-6, c_half_tile = 0.53, f_half_tile = 4.0;
     const int splits_tried[] = {1, 2, 3, 4, 6, 8, 12, 16};
     const int qk = k / rf::BK;
@@ -494,6 +496,17 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
         const long tiles = (long)ceil_div(m, v.bm) * ceil_div(n, v.bn);
         for (int sp : splits_tried) {
             if (sp > qk) break;
+            if (v.k_groups > 1) {
+                if (sp != 1 || qk % v.k_groups != 0) continue;
+                const double t = (double)((tiles + num_cu - 1) / num_cu) * (qk / v.k_groups * cd.c + cd.f);
+                if (t < best_cost) {
+                    best_cost = t;
+                    out->variant = cd.variant;
+                    out->split_k = 1;
+                    out->stream_k = RF_SCHEDULE_TILES;
+                }
+                continue;
+            }
             const int kb_per = ceil_div(qk, sp), splits = ceil_div(qk, kb_per);
             const long rounds = (tiles * splits + num_cu - 1) / num_cu;
             for (int sched : {RF_SCHEDULE_TILES, RF_SCHEDULE_PERSISTENT}) {
