@@ -215,27 +215,52 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
     // ---- two load cursors run ahead of the compute position ----
     // cursor 1 = the K block after the current one (DMA instructions d >= TN, issued in the first slots of a step);
     // cursor 2 = two blocks ahead (instructions d < TN, issued after the barrier). Each holds its tile ordinal, K block
-    // and the running source pointers of its instructions; crossing into the next tile recomputes the pointers from
-    // that tile's origin.
+    // and the source pointers of its instructions; crossing into the next tile recomputes the pointers from that
+    // tile's origin.
+    // BY_OPERAND: the cursors split the instructions by operand (cursor 2 = the A rows, cursor 1 = the B rows and the
+    // scales), so each per-lane offset register belongs to one cursor and can carry that cursor's K position: a step
+    // is then a handful of 32-bit vector adds beside the MFMAs, the scalar pointers stay at the tile's first K block,
+    // and the ten 64-bit scalar additions per K block (a burst of scalar work after the last slot) are gone. The
+    // offsets stay below K * M and K * N, which the host keeps under 2^32 for this kernel.
+    constexpr bool BY_OPERAND = TN == INST_A;
+    const uint32_t step_a = (uint32_t)BK * (uint32_t)M, step_b = (uint32_t)BK * (uint32_t)N, step_s = (uint32_t)M * 4u,
+                   step_sb = (uint32_t)QN * 4u;
     const uint8_t *dsrc[NDMA];
     int c1_r = 0, c1_kb = 0, c2_r = 0, c2_kb = 0;     // set below
-    auto seek = [&](int which, int r, int kb) {        // point a cursor's instructions at (tile r, block kb)
+    auto shift_offsets = [&](int which, int blocks) {  // BY_OPERAND: move a cursor's per-lane offsets by `blocks` K blocks
+        if (which == 2) {
+#pragma unroll
+            for (int c_ = 0; c_ < NCLS_A; c_++) goff_a[c_] += (uint32_t)blocks * step_a;
+        } else {
+#pragma unroll
+            for (int c_ = 0; c_ < NCLS_B; c_++) goff_b[c_] += (uint32_t)blocks * step_b;
+            goff_s += (uint32_t)blocks * step_s;
+            goff_sb += (uint32_t)blocks * step_sb;
+        }
+    };
+    // point a cursor's instructions at (tile r, block kb); from_kb = the block its offsets stand at (BY_OPERAND)
+    auto seek = [&](int which, int r, int kb, int from_kb) {
         int m0, n0;
         tile_origin(r, m0, n0);
 #pragma unroll
         for (int d = 0; d < NDMA; d++)
-            if ((d >= TN) == (which == 1)) dsrc[d] = dma_src(d, m0, n0, kb);
+            if ((d >= TN) == (which == 1)) dsrc[d] = dma_src(d, m0, n0, BY_OPERAND ? 0 : kb);
+        if constexpr (BY_OPERAND) shift_offsets(which, kb - from_kb);
     };
     auto advance = [&](int which, int &r, int &kb) {   // move a cursor one K block on
         if (kb + 1 < QK) {
             kb += 1;
+            if constexpr (BY_OPERAND) {
+                shift_offsets(which, 1);
+            } else {
 #pragma unroll
-            for (int d = 0; d < NDMA; d++)
-                if ((d >= TN) == (which == 1)) dsrc[d] += dma_step(d);
+                for (int d = 0; d < NDMA; d++)
+                    if ((d >= TN) == (which == 1)) dsrc[d] += dma_step(d);
+            }
         } else {
             r += 1;
+            seek(which, r, 0, kb);
             kb = 0;
-            seek(which, r, 0);
         }
     };
 
@@ -255,12 +280,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_fp8_blockscale_per
         // cursor 2 issues its part of block 1 here and moves on to block 2 (or the next tile); cursor 1 stands at
         // block 1 (QK >= 2)
         c2_r = 0; c2_kb = 1;
-        seek(2, 0, 1);
+        seek(2, 0, 1, 0);
 #pragma unroll
         for (int d = 0; d < TN && d < NDMA; d++) issue_dma(d, 1, dsrc[d]);
         advance(2, c2_r, c2_kb);
         c1_r = 0; c1_kb = 1;
-        seek(1, 0, 1);
+        seek(1, 0, 1, 0);
         // like every first K block of a tile, the one that follows finds cursor 1's loads already issued
 #pragma unroll
         for (int d = TN; d < NDMA; d++) issue_dma(d, 1, dsrc[d]);

@@ -391,8 +391,10 @@ bool tiled_path_ok(const void *a, const void *b, const void *c, int m, int n) {
            ((uintptr_t)c % 16) == 0;
 }
 
+// (K * M and K * N below 2^32: the persistent kernel keeps a load cursor's K position in 32-bit per-lane offsets)
 bool persistent_ok(const Variant &v, int m, int n, int k) {
-    return v.persistent && m >= v.bm && m % 16 == 0 && n % v.bn == 0 && (k / rf::BK) % 2 == 0;
+    return v.persistent && m >= v.bm && m % 16 == 0 && n % v.bn == 0 && (k / rf::BK) % 2 == 0 &&
+           (unsigned long long)k * m < (1ull << 32) && (unsigned long long)k * n < (1ull << 32);
 }
 
 // Persistent schedule that finishes the last, partial round with half tiles: one workgroup per CU, at least one whole
