@@ -568,6 +568,39 @@ def main():
             out["operand_bits"][label + "_us"] = round(u, 2)
             del ops
         print("C2 launch time by operand bits: %r" % (out["operand_bits"],), file=sys.stderr)
+        # Calibration only (nothing of the product runs through it): what the vendor's library reaches on the headline
+        # shape for a plain fp8 GEMM WITHOUT block scales (torch._scaled_mm: K-contiguous operands, one scale per tensor
+        # or per row, so no fold per K block), on the same box in the same run. It says what "per cent of the published
+        # peak" means for any fp8 GEMM under this chip's power limit.
+        try:
+            xm = torch.randn((m, k), device="cuda")
+            wm = torch.randn((n, k), device="cuda")
+            cal = {}
+            for label, sx_, sw_ in (("per_tensor_scales", (xm.abs().amax() / 448).float(), (wm.abs().amax() / 448).float()),
+                                    ("per_row_scales", (xm.abs().amax(dim=1, keepdim=True) / 448).float(),
+                                     (wm.abs().amax(dim=1, keepdim=True) / 448).float())):
+                a8_, b8_ = (xm / sx_).to(fp8), (wm / sw_).to(fp8)
+                sb_ = sw_.t() if sw_.dim() == 2 else sw_
+                fn_ = lambda: torch._scaled_mm(a8_, b8_.t(), scale_a=sx_, scale_b=sb_, out_dtype=torch.bfloat16)  # noqa: E731
+                with torch.cuda.stream(stream):
+                    for _ in range(2500):
+                        fn_()
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record(stream)
+                    for _ in range(100):
+                        fn_()
+                    e1.record(stream)
+                    stream.synchronize()
+                u = e0.elapsed_time(e1) * 1e3 / 100
+                cal[label] = {"us": round(u, 2), "tflops": round(flop / u / 1e6, 1),
+                              "pct_fp8_mfma_peak": round(100 * flop / u / 1e6 / PEAK_FP8_TFLOPS, 2)}
+            cal["note"] = ("torch._scaled_mm (the vendor's GEMM library) on %dx%dx%d, fp8 e4m3fn -> bf16, no block scales: "
+                           "calibration of the target only, not a code path of this library" % (m, n, k))
+            out["calibration_vendor_fp8_gemm_without_block_scales"] = cal
+            print("calibration, vendor library, plain fp8 GEMM without block scales: %r" % (cal,), file=sys.stderr)
+            del xm, wm
+        except Exception as e:      # an installation without that routine or format: the calibration is simply absent
+            print("calibration with torch._scaled_mm not available: %s" % str(e)[:200], file=sys.stderr)
         # what the chip sustains on the same MFMA instruction from registers alone (clock under its power limit);
         # run as a child process once the GEMM work above is done
         probe = os.path.join(ROOT, "bench_probes", "mfma_ceiling")
