@@ -101,6 +101,9 @@ const Variant kVariants[] = {
     // the split-K plan of a short, wide-K shape in one launch, with no partial sums in memory
     Variant{64, 128, 2, 2, rf::InWgSplitGeom<64, 128, 2, 2, 3, 2>::LDS_BYTES,
             rf::gemm_fp8_blockscale_tile_ksplit_in_wg<64, 128, 2, 2, 3, 2>, nullptr, nullptr, nullptr, 0, nullptr, 2},
+    // 13: the 128 x 128 two-stage tile with K split between two wave groups (8 waves, 130 KiB LDS)
+    Variant{128, 128, 2, 2, rf::InWgSplitGeom<128, 128, 2, 2, 2, 2>::LDS_BYTES,
+            rf::gemm_fp8_blockscale_tile_ksplit_in_wg<128, 128, 2, 2, 2, 2>, nullptr, nullptr, nullptr, 0, nullptr, 2},
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
@@ -485,10 +488,13 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
     // no padded columns, e.g. N = 576, 1536 or 3072; the 64x128 tile where M is short or the whole problem is a few
     // microseconds); the others never won by more than a few percent.
     struct Candidate { int variant; double c, f; };
-    // (variant 12 splits K between two wave groups of one workgroup: half the K blocks per group, one launch, no reduction
-    // term; fitted on its 103 tabled measurements: the best plan of short shapes, M <= 512, with K = 512 ... 2304)
+    // (variants 12 and 13 split K between two wave groups of one workgroup: half the K blocks per group, one launch, no
+    // reduction term. Variant 12, the 64 x 128 tile, fitted on its 103 tabled measurements: the best plan of short shapes,
+    // M <= 512, with K = 512 ... 2304. Variant 13, the 128 x 128 tile, fitted on eight shapes with M = 256 ... 1024 and
+    // K = 512 ... 2304: the best plan where 128 x 128 tiles fill one round, e.g. 1024 x 3072 x 1536, 512 x 7168 x 2048)
     const Candidate cands[] = {{0, 0.955, 7.96}, {3, 0.619, 5.11}, {5, 0.71, 5.2},  {6, 0.74, 3.7},  {7, 0.82, 0.0},
-                               {8, 0.52, 4.5},   {9, 0.70, 0.5},   {10, 0.53, 5.9}, {11, 0.62, 5.8}, {12, 0.75, 2.9}};
+                               {8, 0.52, 4.5},   {9, 0.70, 0.5},   {10, 0.53, 5.9}, {11, 0.62, 5.8}, {12, 0.75, 2.9},
+                               {13, 1.09, 4.2}};
     const double f_next = 3.0, reduce_fixed = 2.83, reduce_per_elem = 1.37e-6, c_half_tile = 0.53, f_half_tile = 4.0;
     const int splits_tried[] = {1, 2, 3, 4, 6, 8, 12, 16};
     const int qk = k / rf::BK;

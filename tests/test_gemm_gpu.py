@@ -279,7 +279,8 @@ def test_skinny_k_schedule_bit_exact(rfk, m, n, k):
     assert_close_to_oracle(out, oracle_bf16(noisy), RTOL, ATOL, "skinny K")
 
 
-@pytest.mark.parametrize("m,n,k", [(64, 128, 256), (1024, 1536, 7168), (208, 576, 1024), (64, 1536, 7168), (1024, 512, 512)])
+@pytest.mark.parametrize("m,n,k", [(64, 128, 256), (1024, 1536, 7168), (208, 576, 1024), (64, 1536, 7168), (1024, 512, 512),
+                                   (208, 576, 768), (512, 3072, 1536), (128, 128, 384)])
 def test_k_split_inside_the_workgroup_equals_the_two_launch_form(rfk, m, n, k):
     """Variants whose wave groups split K inside one workgroup (partial sums added through LDS in part order) against
     the same tile with split_k = the number of groups (fp32 partial sums through memory + the reduction kernel): the
@@ -294,7 +295,11 @@ def test_k_split_inside_the_workgroup_equals_the_two_launch_form(rfk, m, n, k):
                 and w["lds_bytes"] * v["k_groups"] > v["lds_bytes"] - 4096]
         assert len(twin) == 1, "the one-group variant with the same tile and stage count"
         cfg, cfg2 = rfk.GemmConfig(v["variant"], 1, 8, 0), rfk.GemmConfig(twin[0]["variant"], v["k_groups"], 8, 0)
-        assert (k // 128) % v["k_groups"] == 0
+        if (k // 128) % v["k_groups"] != 0:
+            with pytest.raises(RuntimeError):                   # K blocks the groups do not divide: refused
+                _run(rfk, exact_problem(m, n, k, seed=1), config=cfg)
+            tried += 1
+            continue
         data = exact_problem(m, n, k, seed=m + n + k)
         exp = oracle_bf16(data)
         for rep in range(2):
@@ -307,8 +312,6 @@ def test_k_split_inside_the_workgroup_equals_the_two_launch_form(rfk, m, n, k):
         for bad in (rfk.GemmConfig(v["variant"], 2, 8, 0), rfk.GemmConfig(v["variant"], 1, 8, 2)):
             with pytest.raises(RuntimeError):
                 _run(rfk, data, config=bad)
-        with pytest.raises(RuntimeError):                       # three K blocks, two groups
-            _run(rfk, exact_problem(64, 128, 384, seed=1), config=cfg)
         tried += 1
     assert tried > 0
 
