@@ -183,7 +183,9 @@ void rf_gemm_destroy(void);
  * c is written in place, rows of neighbouring groups are not touched). Ragged N, unaligned b or c, and problems below
  * 2^21 multiply-adds run the bounds-checked kernel once per group.
  * variant: -1 = automatic, else an index into {256x256, 128x256, 128x128, 128x64} tiles, or 4 = 256-row tiles with a
- * 128 x 256 tile for a group's last rows when at most 128 are left. */
+ * 128 x 256 tile for a group's last rows when at most 128 are left, or 5 = 256-row tiles with a last tile of 64, 128,
+ * 192 or 256 rows, run by one resident workgroup per CU that takes tiles from a queue per XCD (the automatic choice
+ * for groups of uneven size; its queues are counters in the stream's buffer set, like the stream-K schedule's). */
 int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const float *bs, void *c, const int *row_offsets,
                         int groups, int n, int k, int variant, hipStream_t stream);
 

@@ -123,7 +123,7 @@ template <int BM, int BN, int WAVES_M, int WAVES_N, int NS = 2>
 __device__ __forceinline__ void tile_mainloop(
     const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
     const float *__restrict__ SB, int M, int ldm, int N, int m0, int n0, int kb_begin, int kb_end, uint8_t *lds,
-    f32x4 (&acc)[BM / WAVES_M / 16][BN / WAVES_N / 16]) {
+    f32x4 (&acc)[BM / WAVES_M / 16][BN / WAVES_N / 16], int opaque_zero = 0) {
     using G = TileGeom<BM, BN, WAVES_M, WAVES_N, NS>;
     constexpr int NW = WAVES_M * WAVES_N;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
@@ -152,7 +152,10 @@ __device__ __forceinline__ void tile_mainloop(
     constexpr int ROWS_W_A = INST_A * 64 / CPR_A, ROWS_W_B = INST_B * 64 / CPR_B;      // rows per wave
     static_assert((INST_A * 64) % CPR_A == 0 && (INST_B * 64) % CPR_B == 0, "a wave's loads cover whole rows");
 
-    const int tid = threadIdx.x;
+    // (opaque_zero: a caller that runs several instantiations of this loop inside a loop of its own passes a zero the
+    // compiler cannot see through, made inside its loop; otherwise every instantiation's per-lane offsets are computed
+    // once before the caller's loop and stay in registers through all of it)
+    const int tid = threadIdx.x + opaque_zero;
     const int lane = tid & 63;
     // (a workgroup may hold several wave groups of NW waves, each running this loop on its own tile of LDS: the wave's
     // index inside its group)
@@ -1016,6 +1019,88 @@ __global__ __launch_bounds__(512) void gemm_fp8_blockscale_grouped_mixed(
         f32x4 acc[TileGeom<128, 256, 2, 4>::TM][TileGeom<128, 256, 2, 4>::TN];
         tile_mainloop<128, 256, 2, 4, 3>(A + r1, Bg, SA + r1, SBg, rest, M_total, N, 0, n0, 0, QK, lds, acc);
         store_tile_bf16<128, 256, 2, 4>(acc, C + (size_t)(out0 + big_m * 256) * N, out_rows - big_m * 256, N, 0, n0, lds);
+    }
+}
+
+// The grouped GEMM with tiles of four heights and work queues. A group's rows are cut into 256-row tiles and one last
+// tile of 64, 128, 192 or 256 rows (the smallest that holds what is left), all 256 columns wide and all run by eight
+// waves: uneven groups pad their rows to a multiple of 64 instead of 128 or 256 (32 groups of 16..816 rows: 9088 rows
+// of MFMA work instead of 10240), and a short tile spends its time on what it has to do anyway, streaming its column
+// tile of the group's weights. Tiles of different heights take different times, so the work is not dealt out by the
+// hardware's dispatcher (which hands out workgroups in id order and makes all XCDs wait for the slowest): one
+// workgroup per CU stays resident and takes items from queues, one queue per XCD. The host puts the items in one
+// line (group after group in an order of its choice; inside a group column tile by column tile, the row tiles of one
+// column tile next to each other) and cuts the line into eight pieces, one per queue: whole groups per queue where
+// there are enough of them, the longest first, so that a group's activations and each of its weight tiles are
+// fetched by one L2 and the short tiles fill the end of the launch. (Column tiles dealt out over the XCDs instead,
+// every queue with the same mix: 6 % slower, every XCD then fetches every group's activations.) A workgroup whose
+// own queue is empty helps with the others' in turn. A queue is one counter in device memory: atomicInc with a wrap
+// value of (items + workgroups - 1). Every workgroup draws from a queue until it draws a number that is no item,
+// exactly once per queue, so the counter's last draw wraps it back to zero: the counters need no clearing between
+// launches (launches that share counters must not overlap).
+// In the table of this kernel tile_start[p] counts the items of the first p groups of the line.
+// ---------------------------------------------------------------------------------------------
+struct GroupQueues {
+    int piece_start[NUM_XCD + 1];        // queue x holds items piece_start[x] .. piece_start[x + 1] - 1 of the line
+    int workgroups;                      // of the launch
+    uint8_t order[kMaxGroups];           // order[p]: the group at position p of the line
+};
+constexpr int kQueueTileLds =
+    TileGeom<256, 256, 2, 4>::LDS_BYTES > TileGeom<128, 256, 2, 4, 3>::LDS_BYTES ? TileGeom<256, 256, 2, 4>::LDS_BYTES
+                                                                                 : TileGeom<128, 256, 2, 4, 3>::LDS_BYTES;
+static_assert(TileGeom<192, 256, 2, 4>::LDS_BYTES <= kQueueTileLds && TileGeom<64, 256, 2, 4, 3>::LDS_BYTES <= kQueueTileLds,
+              "the 256- and 128-row tiles are the largest");
+constexpr int kQueueLds = kQueueTileLds + 16;                    // + the slot through which a draw reaches all waves
+template <int BM, int NS>
+__device__ __forceinline__ void grouped_queue_tile(const uint8_t *A, const uint8_t *B, const float *SA, const float *SB,
+                                                   uint16_t *C, int rows, int out_rows, int M_total, int N, int n0, int QK,
+                                                   uint8_t *lds) {
+    f32x4 acc[TileGeom<BM, 256, 2, 4>::TM][TileGeom<BM, 256, 2, 4>::TN];
+    int vz;
+    asm volatile("v_mov_b32 %0, 0" : "=v"(vz));
+    tile_mainloop<BM, 256, 2, 4, NS>(A, B, SA, SB, rows, M_total, N, 0, n0, 0, QK, lds, acc, vz);
+    store_tile_bf16<BM, 256, 2, 4>(acc, C, out_rows, N, 0, n0, lds);
+}
+__global__ __launch_bounds__(512) void gemm_fp8_blockscale_grouped_queue(
+    const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ SA,
+    const float *__restrict__ SB, uint16_t *__restrict__ C, int M_total, int N, int K, int groups,
+    const GroupTable table, const GroupQueues queues, unsigned *__restrict__ counters) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    volatile int *drawn = (volatile int *)(lds + kQueueTileLds);
+    const int QK = K / BK, QN = (N + 127) / 128;
+    const int xcd = blockIdx.x % NUM_XCD;
+    for (int turn = 0; turn < NUM_XCD; turn++) {
+        const int qx = (xcd + turn) % NUM_XCD;
+        const int first = queues.piece_start[qx], count = queues.piece_start[qx + 1] - first;
+        for (;;) {
+            __syncthreads();             // the previous item's staged stores and the previous draw have been read
+            if (threadIdx.x == 0)
+                *drawn = (int)atomicInc(counters + qx, (unsigned)(count + queues.workgroups - 1));
+            __syncthreads();
+            const int got = __builtin_amdgcn_readfirstlane(*drawn);
+            if (got >= count) break;
+            const int item = first + got;
+            int lo = 0, hi = groups;     // the last p with tile_start[p] <= item (empty groups own no item)
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) >> 1;
+                if (table.tile_start[mid] <= item) lo = mid; else hi = mid;
+            }
+            const int grp = queues.order[lo], local = item - table.tile_start[lo];
+            const int row0 = table.row_start[grp], rows = table.row_start[grp + 1] - row0;
+            const int out0 = table.out_row_start[grp], out_rows = table.out_row_start[grp + 1] - out0;
+            const int full = rows / 256, rest = rows - full * 256;
+            const int tiles_m = full + (rest > 0 ? 1 : 0);
+            const int tile_m = local % tiles_m, n0 = (local / tiles_m) * 256, m0 = tile_m * 256;
+            const int height = tile_m < full ? 4 : (rest + 63) / 64;           // in units of 64 rows
+            const uint8_t *Ai = A + row0 + m0, *Bg = B + (size_t)grp * K * N;
+            const float *SAi = SA + row0 + m0, *SBg = SB + (size_t)grp * QK * QN;
+            uint16_t *Ci = C + (size_t)(out0 + m0) * N;
+            const int r = rows - m0, o = out_rows - m0;
+            if (height == 4) grouped_queue_tile<256, 2>(Ai, Bg, SAi, SBg, Ci, r, o, M_total, N, n0, QK, lds);
+            else if (height == 3) grouped_queue_tile<192, 2>(Ai, Bg, SAi, SBg, Ci, r, o, M_total, N, n0, QK, lds);
+            else if (height == 2) grouped_queue_tile<128, 3>(Ai, Bg, SAi, SBg, Ci, r, o, M_total, N, n0, QK, lds);
+            else grouped_queue_tile<64, 3>(Ai, Bg, SAi, SBg, Ci, r, o, M_total, N, n0, QK, lds);
+        }
     }
 }
 

@@ -1177,23 +1177,27 @@ typedef void (*grouped_kernel_t)(const uint8_t *, const uint8_t *, const float *
 struct GroupedVariant {
     int bm, bn, threads, lds;
     grouped_kernel_t kernel;
-    bool mixed;          // 256-row tiles plus one 128-row tile for a left-over of at most 128 rows
+    bool mixed;          // 256-row tiles plus one shorter tile for what is left over (one 128-row tile for at most 128
+                         // rows; the queue form: 64, 128, 192 or 256 rows)
+    bool queue = false;  // resident workgroups that take tiles from per-XCD queues (gemm_fp8_blockscale_grouped_queue)
     // row tiles of a group of `rows` rows
     int tiles_m(int rows) const {
         if (!mixed) return ceil_div(rows, bm);
         return rows / 256 + (rows % 256 > 0 ? 1 : 0);
     }
-    // estimated cost of row tile i of a group of `rows` rows, in full-height tiles (the 128-row tile that ends a group
-    // of the mixed form runs 0.6 times as long as a 256-row one), and of all row tiles of one column tile
 };
+
 #define RF_GROUPED(BM, BN, WM, WN, NS) \
     GroupedVariant { BM, BN, WM *WN * 64, rf::TileGeom<BM, BN, WM, WN, NS>::LDS_BYTES, rf::gemm_fp8_blockscale_grouped<BM, BN, WM, WN, NS>, false }
 constexpr int kMixedLds = rf::TileGeom<256, 256, 2, 4>::LDS_BYTES > rf::TileGeom<128, 256, 2, 4, 3>::LDS_BYTES
                               ? rf::TileGeom<256, 256, 2, 4>::LDS_BYTES : rf::TileGeom<128, 256, 2, 4, 3>::LDS_BYTES;
 const GroupedVariant kGroupedVariants[] = {
     RF_GROUPED(256, 256, 2, 4, 2), RF_GROUPED(128, 256, 2, 4, 3), RF_GROUPED(128, 128, 2, 2, 2), RF_GROUPED(128, 64, 2, 1, 2),
-    GroupedVariant{256, 256, 512, kMixedLds, rf::gemm_fp8_blockscale_grouped_mixed, true}};
-constexpr int kGroupedMixed = 4;
+    GroupedVariant{256, 256, 512, kMixedLds, rf::gemm_fp8_blockscale_grouped_mixed, true},
+    GroupedVariant{256, 256, 512, rf::kQueueLds, nullptr, true, true}};
+constexpr int kGroupedMixed = 4, kGroupedQueue = 5;
+// Estimated time of a 256-column tile of the queue form by its height in units of 64 rows, relative to a 256-row tile
+constexpr double kQueueTileCost[5] = {0.0, 0.68, 0.75, 0.97, 1.0};
 constexpr int kNumGroupedVariants = sizeof(kGroupedVariants) / sizeof(kGroupedVariants[0]);
 
 long grouped_tiles(const GroupedVariant &v, const int *row_offsets, int groups, int n) {
@@ -1226,7 +1230,10 @@ int grouped_gemm(const void *a, const void *b, const float *as, const float *bs,
     if (rc != RF_OK) return rc;
     if (!s.grouped_attrs_set) {
         for (const GroupedVariant &v : kGroupedVariants)
-            RF_HIP(hipFuncSetAttribute((const void *)v.kernel, hipFuncAttributeMaxDynamicSharedMemorySize, v.lds));
+            if (v.kernel)
+                RF_HIP(hipFuncSetAttribute((const void *)v.kernel, hipFuncAttributeMaxDynamicSharedMemorySize, v.lds));
+        RF_HIP(hipFuncSetAttribute((const void *)rf::gemm_fp8_blockscale_grouped_queue,
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, rf::kQueueLds));
         s.grouped_attrs_set = true;
     }
     const int qk = k / rf::BK, qn = ceil_div(n, 128);
@@ -1334,6 +1341,19 @@ int grouped_gemm(const void *a, const void *b, const float *as, const float *bs,
                 const double t = (full + (frac > 0 ? 0.6 + 0.4 * frac : 0.0)) * cost / (double)items;
                 if (best_t == 0 || t < best_t) { best_t = t; variant = cand; }
             }
+            // The queue form (tiles of 64 to 256 rows, resident workgroups): where its shorter last tiles save at least
+            // 7 % of the rows the chosen tiles compute. Measured against the best of the three above: 32 uneven groups
+            // of 16..816 rows (9088 against 10240 rows) 326 against 350 us, 64 groups of 16..176 rows (8000 against
+            // 10624) 395 against 407; groups that the other tiles fit as well (64 x 128, 32 x 256, 20 x 384 rows) run
+            // 2-5 % slower in it, its items being so long that the last ones leave CUs idle.
+            long rows_chosen = 0, rows_queue = 0;
+            for (int g = 0; g < groups; g++) {
+                const int rows = row_offsets[g + 1] - row_offsets[g];
+                rows_queue += ceil_div(rows, 64) * 64;
+                rows_chosen += variant == 0 ? ceil_div(rows, 256) * 256 : variant == 1 ? ceil_div(rows, 128) * 128
+                               : rows / 256 * 256 + (rows % 256 == 0 ? 0 : rows % 256 <= 128 ? 128 : 256);
+            }
+            if (rows_queue * 100 <= rows_chosen * 93) variant = kGroupedQueue;
         }
     }
     const GroupedVariant &v = kGroupedVariants[variant];
@@ -1344,6 +1364,77 @@ int grouped_gemm(const void *a, const void *b, const float *as, const float *bs,
         tiles += v.tiles_m(row_offsets[g + 1] - row_offsets[g]) * tiles_n;
     }
     for (int g = groups; g <= rf::kMaxGroups; g++) table.tile_start[g] = tiles;
+    if (v.queue) {
+        // The line of items and its eight pieces. Estimated time of a group = column tiles x (256-row tiles + what
+        // its last, shorter tile costs relative to one). With at least two groups per XCD: whole groups per queue,
+        // each group to the queue with the least work so far, the longest group first (so every queue's groups are in
+        // falling order). Fewer groups: the groups as they come, cut where the estimated time reaches each eighth.
+        auto rows_of = [&](int g) { return row_offsets[g + 1] - row_offsets[g]; };
+        auto cost_of_tile = [&](int rows, int i) { return i < rows / 256 ? 1.0 : kQueueTileCost[(rows % 256 + 63) / 64]; };
+        auto cost_of = [&](int g) {
+            return tiles_n * (rows_of(g) / 256 + kQueueTileCost[(rows_of(g) % 256 + 63) / 64]);
+        };
+        rf::GroupQueues queues;
+        std::vector<int> order(groups);
+        for (int g = 0; g < groups; g++) order[g] = g;
+        int piece_groups[rf::NUM_XCD + 1] = {0};          // positions of the line where the pieces start, if whole groups
+        const bool whole_groups = groups >= 2 * rf::NUM_XCD;
+        if (whole_groups) {
+            std::stable_sort(order.begin(), order.end(), [&](int x, int y) { return cost_of(x) > cost_of(y); });
+            std::vector<int> lists[rf::NUM_XCD];
+            double load[rf::NUM_XCD] = {0};
+            for (int g : order) {
+                int least = 0;
+                for (int x = 1; x < rf::NUM_XCD; x++)
+                    if (load[x] < load[least]) least = x;
+                lists[least].push_back(g);
+                load[least] += cost_of(g);
+            }
+            int p = 0;
+            for (int x = 0; x < rf::NUM_XCD; x++) {
+                piece_groups[x] = p;
+                for (int g : lists[x]) order[p++] = g;
+            }
+            piece_groups[rf::NUM_XCD] = p;
+        }
+        int items = 0;
+        for (int p = 0; p < groups; p++) {
+            queues.order[p] = (uint8_t)order[p];
+            table.tile_start[p] = items;
+            items += v.tiles_m(rows_of(order[p])) * tiles_n;
+        }
+        for (int p = groups; p <= rf::kMaxGroups; p++) table.tile_start[p] = items;
+        for (int p = groups; p < rf::kMaxGroups; p++) queues.order[p] = 0;
+        if (whole_groups) {
+            for (int x = 0; x <= rf::NUM_XCD; x++) queues.piece_start[x] = table.tile_start[piece_groups[x]];
+        } else {
+            double total = 0, before = 0;
+            for (int g = 0; g < groups; g++) total += cost_of(g);
+            queues.piece_start[0] = 0;
+            int piece = 1, item = 0;
+            for (int g = 0; g < groups; g++) {
+                const int tm = v.tiles_m(rows_of(g));
+                for (int tn = 0; tn < tiles_n && tm > 0; tn++)
+                    for (int i = 0; i < tm; i++, item++) {
+                        while (piece < rf::NUM_XCD && before >= total * piece / rf::NUM_XCD) queues.piece_start[piece++] = item;
+                        before += cost_of_tile(rows_of(g), i);
+                    }
+            }
+            while (piece <= rf::NUM_XCD) queues.piece_start[piece++] = items;
+        }
+        queues.workgroups = s.num_cu >= rf::NUM_XCD ? s.num_cu / rf::NUM_XCD * rf::NUM_XCD : rf::NUM_XCD;
+        if (tiles < queues.workgroups) queues.workgroups = ceil_div(tiles, rf::NUM_XCD) * rf::NUM_XCD;
+        Mem mem{s};
+        mem.stream = stream;
+        unsigned *counters = nullptr;
+        rc = mem.tile_counters(&counters);
+        if (rc != RF_OK) return rc;
+        hipLaunchKernelGGL(rf::gemm_fp8_blockscale_grouped_queue, dim3(queues.workgroups), dim3(v.threads), v.lds, stream,
+                           (const uint8_t *)a, (const uint8_t *)b, as, bs, (uint16_t *)c, m_rows, n, k, groups, table,
+                           queues, counters);
+        RF_HIP(hipGetLastError());
+        return RF_OK;
+    }
     const int longest = ceil_div(tiles, rf::NUM_XCD);          // every XCD takes an eighth of the tiles, rounded
     hipLaunchKernelGGL(v.kernel, dim3(longest * rf::NUM_XCD), dim3(v.threads), v.lds, stream, (const uint8_t *)a,
                        (const uint8_t *)b, as, bs, (uint16_t *)c, m_rows, n, k, groups, table);

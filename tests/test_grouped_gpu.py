@@ -63,7 +63,7 @@ CASES = [([256, 128, 512, 64], 512, 256), ([16, 0, 48, 400, 0, 32], 576, 384), (
 @pytest.mark.parametrize("rows,n,k", CASES)
 def test_grouped_bit_exact_on_exact_data(rfk, rows, n, k):
     g, offs, exp = _grouped_problem(rows, n, k, seed=11 * n + k, exact=True)
-    for variant in (-1, 0, 1, 2, 3, 4):
+    for variant in (-1, 0, 1, 2, 3, 4, 5):
         g[4].zero_()
         rfk.fp8_mm_grouped(*g[:5], offs, variant=variant)
         torch.cuda.synchronize()
@@ -99,7 +99,7 @@ def test_grouped_any_group_sizes_bit_exact(rfk, rows, n, k):
     """Group sizes that are not multiples of 16 (what token routing produces): A is staged with padded groups, C is
     written in place, so rows of the next group must survive and nothing may land past the end."""
     g, offs, exp = _grouped_problem(rows, n, k, seed=31 + n, exact=True)
-    for variant in (-1, 0, 1, 2, 3, 4):
+    for variant in (-1, 0, 1, 2, 3, 4, 5):
         g[4].fill_(-3.0)
         rfk.fp8_mm_grouped(*g[:5], offs, variant=variant)
         torch.cuda.synchronize()
@@ -215,7 +215,7 @@ def test_grouped_gemm_on_the_padded_layout_equals_the_staged_path(rfk, rows, n, 
         sb = torch.full((groups, k // 128, qn), 0.01, device="cuda").permute(0, 2, 1)
     a_flat, sa_flat = rfk.quantize_a(x)
     a_pad, sa_pad = rfk.quantize_a_grouped(x, offs)
-    for variant in (-1, 0, 1, 2, 3, 4):
+    for variant in (-1, 0, 1, 2, 3, 4, 5):
         buf = torch.full((m_total * n + CANARY,), -7.0, dtype=torch.bfloat16, device="cuda")
         c1 = torch.zeros((m_total, n), dtype=torch.bfloat16, device="cuda")
         c2 = buf[: m_total * n].view(m_total, n)
@@ -226,3 +226,60 @@ def test_grouped_gemm_on_the_padded_layout_equals_the_staged_path(rfk, rows, n, 
         assert torch.equal(c1.view(torch.uint16), c2.view(torch.uint16)), "variant %d" % variant
         assert bool(c1.float().abs().sum() > 0)
         _check_canary(buf, m_total * n)
+
+
+def test_grouped_queue_form_repeats_two_streams_and_graph_replays(rfk):
+    """The queue form (variant 5: resident workgroups that draw tiles from one counter per XCD). Its counters return
+    to zero with the last draw of every launch, so launches of different layouts follow each other on one stream
+    without a clear in between; two streams have their own counters and may overlap; a launch captured into a HIP graph
+    replays to the same bits, with the program's own eager launches between the replays. Layouts: 24 uneven groups
+    (whole groups per queue), 5 groups (the line cut by estimated time), 3 tiles in all (fewer than workgroups)."""
+    layouts = [([int(x) * 16 for x in np.random.default_rng(9).integers(0, 40, 24)], 768, 384),
+               ([272, 16, 640, 0, 128], 512, 256), ([64, 16, 48], 256, 128)]
+    probs = [_grouped_problem(rows, n, k, seed=77 + n, exact=True) for rows, n, k in layouts]
+
+    def launch_and_check(i, stream=None):
+        g, offs, exp = probs[i]
+        g[4].fill_(-5.0)
+        with torch.cuda.stream(stream or torch.cuda.current_stream()):
+            rfk.fp8_mm_grouped(*g[:5], offs, variant=5)
+        return lambda: (np.array_equal(bf16_bits(g[4]), exp), "layout %d" % i)
+
+    for i in (0, 1, 2, 1, 0, 0, 2):                       # one stream, no clear between launches
+        check = launch_and_check(i)
+        torch.cuda.synchronize()
+        ok, what = check()
+        assert ok, what
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    for _ in range(4):                                    # two streams at once, each with its own counters
+        c1, c2 = launch_and_check(0, s1), launch_and_check(1, s2)
+        torch.cuda.synchronize()
+        for ok, what in (c1(), c2()):
+            assert ok, "two streams, " + what
+    g, offs, exp = probs[0]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rfk.fp8_mm_grouped(*g[:5], offs, variant=5)
+    for _ in range(3):
+        g[4].fill_(-5.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(bf16_bits(g[4]), exp), "graph replay"
+        check = launch_and_check(1)                       # eager work between two replays
+        torch.cuda.synchronize()
+        assert check()[0]
+
+
+def test_grouped_uneven_groups_take_the_queue_form_automatically(rfk):
+    """Uneven groups whose last tiles are much shorter than 128 rows: the automatic choice gives the bits of the queue
+    form and of every other form (all compute a row of C with the same operations in the same order)."""
+    rows = [16, 32, 272, 48, 528, 64, 16, 80, 304, 16, 32, 144, 16, 784, 48, 32, 16, 64, 272, 16]
+    g, offs, exp = _grouped_problem(rows, 2048, 256, seed=123, exact=True)
+    for variant in (-1, 5, 1):
+        g[4].zero_()
+        rfk.fp8_mm_grouped(*g[:5], offs, variant=variant)
+        torch.cuda.synchronize()
+        assert np.array_equal(bf16_bits(g[4]), exp), "variant %d" % variant
+    _check_canary(g[5], g[4].numel())
