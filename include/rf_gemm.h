@@ -70,8 +70,8 @@ typedef struct rf_gemm_config {
                                       left-over tiles finished as 128-row half tiles, one per CU; 256x256 tile only,
                                       needs the persistent schedule's shape rules, at least one tile per CU and a
                                       last round that is at most half full;
-                         4 SKINNY_K   K = 128 or 256 only: persistent grid, a workgroup keeps the B operand of a strip of
-                                      256 columns in registers and streams A in items of 128 rows, storing each
+                         4 SKINNY_K   K = 128 ... 512 only: persistent grid, a workgroup keeps the B operand of a strip of
+                                      256 columns in registers and streams A in items of 128 (K > 256: 64) rows, storing each
                                       16-row piece of C as soon as it is complete (the launch is a streaming store of
                                       C); needs variant == 0, split_k == 1, M a multiple of 16, N a multiple of 64 */
 } rf_gemm_config;

@@ -225,6 +225,10 @@ int ensure_device_info(State &s) {
                                rf::SkinnyGeom<1>::LDS_BYTES));
     RF_HIP(hipFuncSetAttribute((const void *)rf::gemm_fp8_blockscale_skinny<2>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                rf::SkinnyGeom<2>::LDS_BYTES));
+    RF_HIP(hipFuncSetAttribute((const void *)rf::gemm_fp8_blockscale_skinny<3>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                               rf::SkinnyGeom<3>::LDS_BYTES));
+    RF_HIP(hipFuncSetAttribute((const void *)rf::gemm_fp8_blockscale_skinny<4>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                               rf::SkinnyGeom<4>::LDS_BYTES));
     // the device address of this device's copy of the scratch array (the array's name is only a host-side handle)
     void *scratch_ptr = nullptr;
     RF_HIP(hipGetSymbolAddress(&scratch_ptr, HIP_SYMBOL(scratch)));
@@ -409,9 +413,9 @@ bool half_tail_ok(const Variant &v, int m, int n, int k, int num_cu) {
     return t >= num_cu && r > 0 && (r + 7) / 8 * 8 + r <= num_cu;
 }
 
-// Skinny-K schedule (fp8_gemm_skinny.h): one or two K blocks, whole 16-row m-tiles and whole 64-column wave tiles.
+// Skinny-K schedule (fp8_gemm_skinny.h): one to four K blocks, whole 16-row m-tiles and whole 64-column wave tiles.
 bool skinny_ok(int m, int n, int k) {
-    return (k == rf::BK || k == 2 * rf::BK) && m >= 16 && m % 16 == 0 && n >= 64 && n % 64 == 0;
+    return k >= rf::BK && k <= 4 * rf::BK && k % rf::BK == 0 && m >= 16 && m % 16 == 0 && n >= 64 && n % 64 == 0;
 }
 
 // Stream-K: at least one tile per workgroup (then a split tile has exactly two contributors, which is all the kernel
@@ -465,11 +469,16 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
         out->stream_k = hit->stream_k;
         return;
     }
-    // One or two K blocks and a large C: the launch is a streaming store, which the skinny-K schedule does best
+    // Up to four K blocks and a large C: the launch is a streaming store, which the skinny-K schedule does best
     // (measured against the best tiled plan at N = 7168, K = 256: 1024 rows 6.5 against 6.9 us, 2048 rows 7.8 against
     // 10.3, 6144 rows 18.2 against 22.1; below about six million outputs the 64 x 128 tiles win, e.g. 2048 x 2048: 6.5
-    // against 5.6 us).
-    if (skinny_ok(m, n, k) && (double)m * n >= 6.0e6) {
+    // against 5.6 us). Three and four K blocks (items of 64 rows): from two million outputs on; N = 4096, K = 512: 1024
+    // rows 5.9 against 6.8 us, 4096 rows 12.3 against 13.8, 8192 rows 22.5 against 24.0; N = 7168, K = 384: 512 rows
+    // 4.9 against 6.0, 6144 rows 25.7 against 31.8. With K = 512 and more than sixteen strips the tiled plans are as
+    // fast or faster (N = 7168: 2048 rows 15.1 against 13.1 us, 6144 rows 30.6 against 30.4).
+    if (skinny_ok(m, n, k) &&
+        (k <= 2 * rf::BK ? (double)m * n >= 6.0e6
+                         : (double)m * n >= 2.0e6 && (k == 3 * rf::BK || ceil_div(n, 256) <= 16))) {
         out->variant = 0;
         out->stream_k = RF_SCHEDULE_SKINNY_K;
         return;
@@ -575,7 +584,7 @@ int launch_locked(State &s, Mem &mem, const void *a, const void *b, const float 
                                                "is at most half full");
         } else if (cfg.stream_k == RF_SCHEDULE_SKINNY_K) {
             if (cfg.variant != 0 || !skinny_ok(m, n, k))
-                return fail(RF_ERR_BAD_CONFIG, "the skinny-K schedule needs variant 0, K = 128 or 256, M a multiple of 16 and N a multiple of 64");
+                return fail(RF_ERR_BAD_CONFIG, "the skinny-K schedule needs variant 0, K = 128 ... 512, M a multiple of 16 and N a multiple of 64");
         } else if (cfg.stream_k != RF_SCHEDULE_TILES) {
             return fail(RF_ERR_BAD_CONFIG, "unknown schedule");
         }
@@ -632,14 +641,15 @@ int launch_locked(State &s, Mem &mem, const void *a, const void *b, const float 
         const int strips = ceil_div(n, 256), units = ceil_div(m, 64);
         int per_strip = s.num_cu / strips;
         per_strip = per_strip < 1 ? 1 : per_strip > units ? units : per_strip;
-        if (qk == 1)
-            hipLaunchKernelGGL(rf::gemm_fp8_blockscale_skinny<1>, dim3(strips * per_strip), dim3(512),
-                               rf::SkinnyGeom<1>::LDS_BYTES, stream, (const uint8_t *)a, (const uint8_t *)b, as, bs,
-                               (uint16_t *)c, m, n, per_strip, m_store);
-        else
-            hipLaunchKernelGGL(rf::gemm_fp8_blockscale_skinny<2>, dim3(strips * per_strip), dim3(512),
-                               rf::SkinnyGeom<2>::LDS_BYTES, stream, (const uint8_t *)a, (const uint8_t *)b, as, bs,
-                               (uint16_t *)c, m, n, per_strip, m_store);
+#define RF_LAUNCH_SKINNY(QK)                                                                                            \
+    hipLaunchKernelGGL(rf::gemm_fp8_blockscale_skinny<QK>, dim3(strips * per_strip), dim3(512),                         \
+                       rf::SkinnyGeom<QK>::LDS_BYTES, stream, (const uint8_t *)a, (const uint8_t *)b, as, bs,           \
+                       (uint16_t *)c, m, n, per_strip, m_store)
+        if (qk == 1) RF_LAUNCH_SKINNY(1);
+        else if (qk == 2) RF_LAUNCH_SKINNY(2);
+        else if (qk == 3) RF_LAUNCH_SKINNY(3);
+        else RF_LAUNCH_SKINNY(4);
+#undef RF_LAUNCH_SKINNY
         RF_HIP(hipGetLastError());
         return RF_OK;
     }

@@ -22,7 +22,7 @@ RF_OK = 0
 
 class GemmConfig(ctypes.Structure):
     """rf_gemm_config of include/rf_gemm.h. stream_k is the schedule: 0 one workgroup per tile (and K split),
-    1 stream-K, 2 persistent, 3 persistent with a last round of half tiles, 4 skinny K (K = 128 or 256, variant 0)."""
+    1 stream-K, 2 persistent, 3 persistent with a last round of half tiles, 4 skinny K (K = 128 ... 512, variant 0)."""
     _fields_ = [("variant", ctypes.c_int), ("split_k", ctypes.c_int), ("group_m", ctypes.c_int),
                 ("stream_k", ctypes.c_int)]
 

@@ -78,7 +78,7 @@ def tune_shape(rfk, m, n, k, log=print):
     for v in rfk.variants():
         tiles = -(-m // v["block_m"]) * -(-n // v["block_n"])
         # schedules: 0 = one workgroup per tile (with K splits), 1 = stream-K, 2 = persistent whole tiles,
-        # 3 = persistent with a last round of half tiles, 4 = skinny K (K = 128 or 256; listed under variant 0)
+        # 3 = persistent with a last round of half tiles, 4 = skinny K (K = 128 ... 512; listed under variant 0)
         for split, sk in [(sp, 0) for sp in SPLITS] + [(1, 1), (1, 2), (1, 3), (1, 4)]:
             if split > k // 128 or (sk == 1 and (tiles < ncu or not v["stream_k"])):
                 continue
@@ -86,7 +86,7 @@ def tune_shape(rfk, m, n, k, log=print):
                 continue
             if sk in (2, 3) and (not v["persistent"] or m < v["block_m"] or m % 16 or n % v["block_n"] or (k // 128) % 2):
                 continue
-            if sk == 4 and (v["variant"] != 0 or k > 256 or m % 16 or n % 64):
+            if sk == 4 and (v["variant"] != 0 or k > 512 or m % 16 or n % 64):
                 continue
             if sk == 3:
                 left = tiles % ncu

@@ -148,7 +148,7 @@ def test_compiled_in_plan_table_only_holds_plans_its_shapes_can_run():
         assert m % 16 == 0 and n % 16 == 0 and k % 128 == 0 and 1 <= split <= k // 128 and group >= 1
         assert schedule in (0, 2, 3, 4), "the stream-K schedule is never tabled"
         if schedule == 4:
-            assert variant == 0 and split == 1 and k in (128, 256) and n % 64 == 0
+            assert variant == 0 and split == 1 and k in (128, 256, 384, 512) and n % 64 == 0
         if schedule in (2, 3):
             assert L.rf_gemm_variant_has_persistent(variant) == 1 and split == 1
             assert m >= bm.value and n % bn.value == 0 and (k // 128) % 2 == 0

@@ -259,11 +259,14 @@ def test_half_tile_schedule_rejects_shapes_it_does_not_fit(rfk):
 
 
 @pytest.mark.parametrize("m,n,k", [(128, 256, 256), (16, 64, 128), (272, 320, 256), (1040, 448, 128), (2048, 2048, 256),
-                                   (6000, 7168, 256), (96, 7168, 256), (400, 1216, 256)])
+                                   (6000, 7168, 256), (96, 7168, 256), (400, 1216, 256),
+                                   (64, 256, 512), (16, 64, 384), (272, 320, 512), (1040, 448, 384), (4096, 4096, 512),
+                                   (6000, 4096, 384), (80, 7168, 512), (400, 1216, 512)])
 def test_skinny_k_schedule_bit_exact(rfk, m, n, k):
-    """K = 128 or 256 under the skinny-K schedule (the B operand of a 256-column strip in registers, A streamed in
-    items of 128 rows, C stored m-tile by m-tile): strips that end in a partial 64-column wave tile, a last item with
-    fewer than 128 rows, one to many items and strips per workgroup. Exact data against the oracle, bit for bit, twice
+    """K = 128 ... 512 under the skinny-K schedule (the B operand of a 256-column strip in registers, A streamed in
+    items of 128 rows, 64 rows from three K blocks on, C stored m-tile by m-tile): strips that end in a partial
+    64-column wave tile, a last item with fewer rows, one to many items and strips per workgroup. Exact data against
+    the oracle, bit for bit, twice
     on the same buffers with the canary intact; then data with rounding in it against the one-workgroup-per-tile
     kernel, bit for bit as well (same MFMA, same folds in the same K order)."""
     cfg = rfk.GemmConfig(0, 1, 8, 4)
@@ -317,7 +320,7 @@ def test_k_split_inside_the_workgroup_equals_the_two_launch_form(rfk, m, n, k):
 
 
 def test_skinny_k_schedule_rejects_shapes_it_does_not_fit(rfk):
-    for (m, n, k, variant) in ((256, 256, 384, 0), (256, 256, 512, 0), (40, 256, 256, 0), (256, 96, 256, 0), (256, 256, 256, 1)):
+    for (m, n, k, variant) in ((256, 256, 640, 0), (256, 256, 1024, 0), (40, 256, 256, 0), (256, 96, 256, 0), (256, 256, 256, 1)):
         data = exact_problem(m, n, k, seed=1)
         with pytest.raises(RuntimeError):
             _run(rfk, data, config=rfk.GemmConfig(variant, 1, 8, 4))
