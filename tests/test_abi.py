@@ -178,7 +178,7 @@ def test_planner_arithmetic_on_the_host_for_any_compute_unit_count(tmp_path):
     the table (measured on 256) is left aside and the cost model counts rounds for the count given: every plan names an
     existing variant and a split that leaves each part a K block, the persistent schedules only where the shape allows
     them, the half-tile schedule only when the last round of 256 x 256 tiles on that many units is at most half full,
-    never stream-K, and the skinny-K schedule for one or two K blocks with a large C whatever the count. A loaded plan
+    never stream-K, and the skinny-K schedule for up to four K blocks with a large C whatever the count. A loaded plan
     file still wins on every count."""
     import radeonflow_kernels_amd as rfk
     inc = os.path.join(ROOT, "radeonflow_kernels_amd", "csrc", "tuned_plans.inc")
@@ -201,9 +201,14 @@ def test_planner_arithmetic_on_the_host_for_any_compute_unit_count(tmp_path):
                 left = tiles % ncu
                 assert c.variant == 0 and tiles >= ncu and 0 < left and (left + 7) // 8 * 8 + left <= ncu
             if c.stream_k == 4:
-                assert k in (128, 256) and m % 16 == 0 and n % 64 == 0
+                assert k in (128, 256, 384, 512) and m % 16 == 0 and n % 64 == 0
         assert rfk.plan_for(6144, 7168, 256, ncu).stream_k == 4
         assert rfk.plan_for(2048, 2048, 256, ncu).stream_k != 4            # below six million outputs
+        assert rfk.plan_for(4096, 4096, 512, ncu).stream_k == 4            # three or four K blocks: from two million on
+        assert rfk.plan_for(6144, 7168, 384, ncu).stream_k == 4
+        assert rfk.plan_for(6144, 7168, 512, ncu).stream_k != 4            # K = 512: up to sixteen strips only
+        assert rfk.plan_for(512, 2048, 512, ncu).stream_k != 4
+        assert rfk.plan_for(4096, 4096, 640, ncu).stream_k != 4
     # fewer units, more rounds: 2048 x 2048 x 7168 is 64 tiles of 256 x 256: no K split is worth it on 8 units
     assert rfk.plan_for(2048, 2048, 7168, 8).split_k == 1
     # ragged shapes are planned at their padded size
