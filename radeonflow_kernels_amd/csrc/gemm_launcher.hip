@@ -74,8 +74,8 @@ struct Variant {
               rf::gemm_fp8_blockscale_tile<BM, BN, WM, WN, true>, nullptr, nullptr, 0 }
 // the same with three LDS stages: two K blocks in flight instead of one. A K block of these tiles is 0.4 us of MFMAs,
 // less than a load takes to come back from L2 or the Infinity Cache on a busy chip, so with two stages the loop ran at
-// the latency of its loads: 1024 x 4608 x 7168 45.6 -> 39.0 us, 256 x 7168 x 2304 15.6 -> 13.1 us; the best plan of 54
-// of the 103 tabled shapes. The two-stage forms stay: they fit more workgroups per CU (64 x 128: three instead of
+// the latency of its loads: 1024 x 4608 x 7168 45.6 -> 39.0 us, 256 x 7168 x 2304 15.6 -> 13.1 us; the best plan of 86
+// of the 163 tabled shapes. The two-stage forms stay: they fit more workgroups per CU (64 x 128: three instead of
 // two), which the smallest problems prefer. (128 x 128 with three stages never won and is not built.)
 #define RF_VARIANT_TILE_ONLY_NS3(BM, BN, WM, WN)                                           \
     Variant { BM, BN, WM, WN, rf::TileGeom<BM, BN, WM, WN, 3>::LDS_BYTES,                  \
@@ -484,9 +484,10 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
         return;
     }
     // No measured entry: a cost model whose constants were searched on the tuner's measurements of the tabled shapes so
-    // that its plan comes close to the best measured one (on those 103 shapes, with the skinny-K rule above: 0.8 % slower
-    // on average, 8 % at worst; on 14 shapes outside the table 1.7 % and 7.5 %; the constants rank plans, they are not
-    // measured times). Time in microseconds of a plan =
+    // that its plan comes close to the best measured one (on those 163 shapes, with the skinny-K rule above: 0.8 % slower
+    // on average, 8 % at worst; constants searched on 103 of them were 1.8 % and 16 % behind on the other 60, and 1.7 %
+    // and 7.5 % on 14 shapes outside the table; the constants rank plans, they are not measured times). Time in
+    // microseconds of a plan =
     //   rounds * (K blocks per workgroup * c + f)           one workgroup per tile and K split
     //   rounds * K blocks * c + f + (rounds - 1) * f_next   persistent: only the first tile starts cold
     //   the same over the whole rounds + f_next + K blocks * c + f of the three-stage 128x256 tile
@@ -500,13 +501,13 @@ void select_config(int m, int n, int k, int num_cu, bool tiled_ok, const std::ve
     // microseconds); the others never won by more than a few percent.
     struct Candidate { int variant; double c, f; };
     // (variants 12 and 13 split K between two wave groups of one workgroup: half the K blocks per group, one launch, no
-    // reduction term. Variant 12, the 64 x 128 tile, fitted on its 103 tabled measurements: the best plan of short shapes,
-    // M <= 512, with K = 512 ... 2304. Variant 13, the 128 x 128 tile, fitted on eight shapes with M = 256 ... 1024 and
-    // K = 512 ... 2304: the best plan where 128 x 128 tiles fill one round, e.g. 1024 x 3072 x 1536, 512 x 7168 x 2048)
-    const Candidate cands[] = {{0, 0.805, 6.96}, {3, 0.619, 5.71}, {5, 0.71, 5.2},  {6, 0.74, 3.7},  {7, 0.85, 0.3},
-                               {8, 0.52, 5.1},   {9, 0.82, 0.5},   {10, 0.59, 5.6}, {11, 0.59, 5.8}, {12, 0.84, 2.0},
+    // reduction term. Variant 12, the 64 x 128 tile: the best plan of short shapes, M <= 512, with K = 512 ... 2304.
+    // Variant 13, the 128 x 128 tile: the best plan where 128 x 128 tiles fill one round, e.g. 1024 x 3072 x 1536,
+    // 512 x 7168 x 2048)
+    const Candidate cands[] = {{0, 0.905, 7.46}, {3, 0.619, 5.71}, {5, 0.71, 5.2},  {6, 0.74, 3.7},  {7, 0.91, 0.0},
+                               {8, 0.52, 4.5},   {9, 0.79, 0.5},   {10, 0.53, 5.9}, {11, 0.65, 6.4}, {12, 0.90, 1.7},
                                {13, 1.06, 3.9}};
-    const double f_next = 3.3, reduce_fixed = 4.43, reduce_per_elem = 1.37e-6, c_half_tile = 0.59, f_half_tile = 4.6;
+    const double f_next = 3.3, reduce_fixed = 4.83, reduce_per_elem = 1.37e-6, c_half_tile = 0.47, f_half_tile = 5.2;
     const int splits_tried[] = {1, 2, 3, 4, 6, 8, 12, 16};
     const int qk = k / rf::BK;
     double best_cost = 1e30;

@@ -35,7 +35,7 @@ SHAPES = [
     (96, 4608, 7168), (128, 7168, 2304), (128, 512, 7168), (512, 4096, 512), (512, 1536, 7168),
 ]
 # token counts a server sees, over the (N, K) pairs of the shapes above (--extended)
-EXTENDED_M = (16, 32, 64, 128, 256, 512, 1024, 2048, 4096, 8192)
+EXTENDED_M = (16, 32, 48, 64, 96, 128, 192, 256, 384, 512, 768, 1024, 1536, 2048, 3072, 4096, 6144, 8192)
 EXTENDED = [(m, n, k) for (n, k) in sorted({(n, k) for _, n, k in SHAPES if (n, k) != (64, 128)}) for m in EXTENDED_M
             if (m, n, k) not in SHAPES]
 SPLITS = (1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 16)
