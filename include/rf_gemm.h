@@ -189,6 +189,12 @@ void rf_gemm_destroy(void);
 int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const float *bs, void *c, const int *row_offsets,
                         int groups, int n, int k, int variant, hipStream_t stream);
 
+/* The tile form rf_fp8_gemm_grouped takes with variant = -1 for groups of these sizes on a device with num_cu compute
+ * units (an index as described above); host arithmetic only, no device needed. For launches that take the tiled
+ * kernels (N % 16 == 0, aligned b and c, not a tiny problem). No counterpart in the reference, whose grouped GEMM is
+ * hipBLASLt's (src/moe/moe.cpp:213-221). */
+int rf_grouped_variant_for(const int *row_offsets, int groups, int n, int k, int num_cu, int *variant);
+
 /* The grouped form without the staging copy: a and as already hold every group from a multiple of 16 rows on.
  *   padded_offsets[g] = sum over earlier groups of their row counts rounded up to 16 (rf_grouped_padded_offsets writes
  *   groups + 1 of them on the host; M_pad = padded_offsets[groups]);

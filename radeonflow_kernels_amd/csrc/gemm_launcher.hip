@@ -1221,6 +1221,70 @@ long grouped_tiles(const GroupedVariant &v, const int *row_offsets, int groups, 
 }  // namespace
 
 namespace {
+// The automatic choice of rf_fp8_gemm_grouped (variant = -1) for groups of these sizes on a device with num_cu compute units.
+int choose_grouped_variant(const int *row_offsets, int groups, int n, int k, int num_cu) {
+    // the largest tile that still gives every CU a workgroup; failing that, the one with the most workgroups
+    int variant = -1;
+    long most = -1;
+    int most_v = 0;
+    for (int v = 0; v < kNumGroupedVariants && variant < 0; v++) {
+        const long t = grouped_tiles(kGroupedVariants[v], row_offsets, groups, n);
+        if (t >= num_cu) variant = v;
+        if (t > most) { most = t; most_v = v; }
+    }
+    if (variant < 0) variant = most_v;
+    if (variant == 1) variant = 0;      // 128-row tiles fill the chip: the 256-wide family, chosen below
+    // Enough tiles for the 256-wide family (128-row tiles would give every CU one): 256-row tiles, 128-row tiles
+    // (three stages) or the mixed form, by a
+    // small model of what was measured (N = 4096, K = 7168, twelve group layouts). A tile costs its compute
+    // (91 for 256 rows, 52 for 128, arbitrary units) plus a share of streaming its column tile of the group's
+    // weights (36, divided among the row tiles that use it: they run side by side on one XCD); the launch takes
+    // as many rounds of one tile per CU as the tile count needs, a last partial round counting 0.6 + 0.4 x its
+    // fill. Round counts decide most cases: 32 uneven groups of 16..816 rows are 816 mixed tiles (3.19 rounds,
+    // 369 us) or 1280 tiles of 128 rows (5.00 rounds, 342 us); 20 groups of 384 rows 287 against 246 us; 64 groups
+    // of 16..176 rows 408 against 447 us. On the twelve layouts the choice is 0.9 % slower than the best of the
+    // three on average, 8 % at worst (always taking the mixed form: 2.6 % and 17 %).
+    if (variant == 0) {
+        const int tiles_n256 = ceil_div(n, 256);
+        double best_t = 0;
+        for (int cand : {0, 1, kGroupedMixed}) {
+            double cost = 0;
+            long items = 0;
+            for (int g = 0; g < groups; g++) {
+                const int rows = row_offsets[g + 1] - row_offsets[g];
+                if (rows == 0) continue;
+                int big, small;
+                if (cand == 0) { big = ceil_div(rows, 256); small = 0; }
+                else if (cand == 1) { big = 0; small = ceil_div(rows, 128); }
+                else { big = rows / 256 + (rows % 256 > 128 ? 1 : 0); small = rows % 256 > 0 && rows % 256 <= 128 ? 1 : 0; }
+                cost += tiles_n256 * (91.0 * big + 52.0 * small + 36.0);      // 36 / t for each of the t row tiles
+                items += (long)tiles_n256 * (big + small);
+            }
+            const double rounds_exact = (double)items / num_cu;
+            const double full = std::floor(rounds_exact), frac = rounds_exact - full;
+            const double t = (full + (frac > 0 ? 0.6 + 0.4 * frac : 0.0)) * cost / (double)items;
+            if (best_t == 0 || t < best_t) { best_t = t; variant = cand; }
+        }
+        // The queue form (tiles of 64 to 256 rows, resident workgroups): where its shorter last tiles save at least
+        // 7 % of the rows the chosen tiles compute and it has enough items to go round (1.5 per CU; 2.5 when K is
+        // below 4096 and an item is short against the cost of drawing it). Measured on 68 layouts (8 to 128 groups of
+        // uniform, exponential or equal sizes; N x K = 4096 x 7168, 7168 x 2048, 2048 x 7168, 4096 x 2048) against
+        // the best of the four 256-wide forms: this rule 0.8 % behind on average, 11 % at worst; never the queue form
+        // 4.6 % and 16 %; the queue form on row savings alone 2.2 % and 41 % (16 groups of 16..384 rows at
+        // N = 2048: 170 items for 256 CUs, 91 against 65 us with 128-row tiles).
+        long rows_chosen = 0, rows_queue = 0, items_queue = 0;
+        for (int g = 0; g < groups; g++) {
+            const int rows = row_offsets[g + 1] - row_offsets[g];
+            rows_queue += ceil_div(rows, 64) * 64;
+            items_queue += (long)ceil_div(rows, 256) * tiles_n256;
+            rows_chosen += variant == 0 ? ceil_div(rows, 256) * 256 : variant == 1 ? ceil_div(rows, 128) * 128
+                           : rows / 256 * 256 + (rows % 256 == 0 ? 0 : rows % 256 <= 128 ? 128 : 256);
+        }
+        const long items_needed = k >= 4096 ? 3L * num_cu / 2 : 5L * num_cu / 2;
+        if (rows_queue * 100 <= rows_chosen * 93 && items_queue >= items_needed) variant = kGroupedQueue;
+    }
+    return variant;
+}
 // prepadded: a and as already hold every group from a multiple of 16 rows on (the layout rf_quantize_a_grouped_* writes
 // and rf_grouped_padded_offsets describes); otherwise they hold the groups back to back as row_offsets says.
 int grouped_gemm(const void *a, const void *b, const float *as, const float *bs, void *c, const int *row_offsets,
@@ -1311,64 +1375,7 @@ int grouped_gemm(const void *a, const void *b, const float *as, const float *bs,
         for (int g = 0; g <= rf::kMaxGroups; g++)
             table.row_start[g] = table.out_row_start[g] = row_offsets[g < groups ? g : groups];
     }
-    if (variant < 0) {
-        // the largest tile that still gives every CU a workgroup; failing that, the one with the most workgroups
-        variant = -1;
-        long most = -1;
-        int most_v = 0;
-        for (int v = 0; v < kNumGroupedVariants && variant < 0; v++) {
-            const long t = grouped_tiles(kGroupedVariants[v], row_offsets, groups, n);
-            if (t >= s.num_cu) variant = v;
-            if (t > most) { most = t; most_v = v; }
-        }
-        if (variant < 0) variant = most_v;
-        if (variant == 1) variant = 0;      // 128-row tiles fill the chip: the 256-wide family, chosen below
-        // Enough tiles for the 256-wide family (128-row tiles would give every CU one): 256-row tiles, 128-row tiles
-        // (three stages) or the mixed form, by a
-        // small model of what was measured (N = 4096, K = 7168, twelve group layouts). A tile costs its compute
-        // (91 for 256 rows, 52 for 128, arbitrary units) plus a share of streaming its column tile of the group's
-        // weights (36, divided among the row tiles that use it: they run side by side on one XCD); the launch takes
-        // as many rounds of one tile per CU as the tile count needs, a last partial round counting 0.6 + 0.4 x its
-        // fill. Round counts decide most cases: 32 uneven groups of 16..816 rows are 816 mixed tiles (3.19 rounds,
-        // 369 us) or 1280 tiles of 128 rows (5.00 rounds, 342 us); 20 groups of 384 rows 287 against 246 us; 64 groups
-        // of 16..176 rows 408 against 447 us. On the twelve layouts the choice is 0.9 % slower than the best of the
-        // three on average, 8 % at worst (always taking the mixed form: 2.6 % and 17 %).
-        if (variant == 0) {
-            const int tiles_n256 = ceil_div(n, 256);
-            double best_t = 0;
-            for (int cand : {0, 1, kGroupedMixed}) {
-                double cost = 0;
-                long items = 0;
-                for (int g = 0; g < groups; g++) {
-                    const int rows = row_offsets[g + 1] - row_offsets[g];
-                    if (rows == 0) continue;
-                    int big, small;
-                    if (cand == 0) { big = ceil_div(rows, 256); small = 0; }
-                    else if (cand == 1) { big = 0; small = ceil_div(rows, 128); }
-                    else { big = rows / 256 + (rows % 256 > 128 ? 1 : 0); small = rows % 256 > 0 && rows % 256 <= 128 ? 1 : 0; }
-                    cost += tiles_n256 * (91.0 * big + 52.0 * small + 36.0);      // 36 / t for each of the t row tiles
-                    items += (long)tiles_n256 * (big + small);
-                }
-                const double rounds_exact = (double)items / s.num_cu;
-                const double full = std::floor(rounds_exact), frac = rounds_exact - full;
-                const double t = (full + (frac > 0 ? 0.6 + 0.4 * frac : 0.0)) * cost / (double)items;
-                if (best_t == 0 || t < best_t) { best_t = t; variant = cand; }
-            }
-            // The queue form (tiles of 64 to 256 rows, resident workgroups): where its shorter last tiles save at least
-            // 7 % of the rows the chosen tiles compute. Measured against the best of the three above: 32 uneven groups
-            // of 16..816 rows (9088 against 10240 rows) 326 against 350 us, 64 groups of 16..176 rows (8000 against
-            // 10624) 395 against 407; groups that the other tiles fit as well (64 x 128, 32 x 256, 20 x 384 rows) run
-            // 2-5 % slower in it, its items being so long that the last ones leave CUs idle.
-            long rows_chosen = 0, rows_queue = 0;
-            for (int g = 0; g < groups; g++) {
-                const int rows = row_offsets[g + 1] - row_offsets[g];
-                rows_queue += ceil_div(rows, 64) * 64;
-                rows_chosen += variant == 0 ? ceil_div(rows, 256) * 256 : variant == 1 ? ceil_div(rows, 128) * 128
-                               : rows / 256 * 256 + (rows % 256 == 0 ? 0 : rows % 256 <= 128 ? 128 : 256);
-            }
-            if (rows_queue * 100 <= rows_chosen * 93) variant = kGroupedQueue;
-        }
-    }
+    if (variant < 0) variant = choose_grouped_variant(row_offsets, groups, n, k, s.num_cu);
     const GroupedVariant &v = kGroupedVariants[variant];
     const int tiles_n = ceil_div(n, v.bn);
     int tiles = 0;
@@ -1502,6 +1509,18 @@ int rf_fp8_gemm_grouped(const void *a, const void *b, const float *as, const flo
 int rf_fp8_gemm_grouped_padded(const void *a, const void *b, const float *as, const float *bs, void *c,
                                const int *row_offsets, int groups, int n, int k, int variant, hipStream_t stream) {
     return grouped_gemm(a, b, as, bs, c, row_offsets, groups, n, k, variant, stream, true);
+}
+
+int rf_grouped_variant_for(const int *row_offsets, int groups, int n, int k, int num_cu, int *variant) {
+    g_last_error.clear();
+    if (!row_offsets || !variant) return fail(RF_ERR_NULL_POINTER, "row_offsets or variant is null");
+    if (groups < 1 || groups > rf::kMaxGroups || n < 1 || k < rf::BK || k % rf::BK != 0 || num_cu < 1 || row_offsets[0] != 0)
+        return fail(RF_ERR_BAD_SHAPE, "unsupported shape (need 1 <= groups <= 256, N >= 1, K a positive multiple of 128, "
+                                      "a compute unit count, row_offsets[0] == 0)");
+    for (int g = 0; g < groups; g++)
+        if (row_offsets[g + 1] < row_offsets[g]) return fail(RF_ERR_BAD_SHAPE, "row_offsets must not decrease");
+    *variant = choose_grouped_variant(row_offsets, groups, n, k, num_cu);
+    return RF_OK;
 }
 
 int rf_grouped_padded_offsets(const int *row_offsets, int groups, int *padded_offsets) {

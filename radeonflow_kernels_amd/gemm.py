@@ -44,7 +44,8 @@ EXPORTS = ("run", "rf_fp8_gemm", "rf_fp8_gemm_ex", "rf_gemm_select_config", "rf_
            "rf_gemm_last_error", "rf_fp8_gemm_grouped", "rf_quantize_a_f32", "rf_quantize_a_bf16", "rf_quantize_b_f32", "rf_quantize_b_bf16",
            "rf_cast_f32_to_e4m3fn", "rf_gemm_load_plans", "rf_gemm_clear_plans", "rf_fp8_gemm_time", "rf_fp8_gemm_static",
            "rf_gemm_static_scratch_bytes", "rf_grouped_padded_offsets", "rf_quantize_a_grouped_f32",
-           "rf_quantize_a_grouped_bf16", "rf_fp8_gemm_grouped_padded", "rf_gemm_plan_for", "rf_gemm_variant_k_groups")
+           "rf_quantize_a_grouped_bf16", "rf_fp8_gemm_grouped_padded", "rf_gemm_plan_for", "rf_gemm_variant_k_groups",
+           "rf_grouped_variant_for")
 
 
 def lib():
@@ -97,6 +98,8 @@ def lib():
         L.rf_fp8_gemm_grouped_padded.restype = i32
         L.rf_grouped_padded_offsets.argtypes = [ctypes.POINTER(i32), i32, ctypes.POINTER(i32)]
         L.rf_grouped_padded_offsets.restype = i32
+        L.rf_grouped_variant_for.argtypes = [ctypes.POINTER(i32), i32, i32, i32, i32, ctypes.POINTER(i32)]
+        L.rf_grouped_variant_for.restype = i32
         for name in ("rf_quantize_a_grouped_f32", "rf_quantize_a_grouped_bf16"):
             f = getattr(L, name)
             f.argtypes = [ctypes.c_void_p, ctypes.POINTER(i32), i32, i32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
@@ -201,6 +204,19 @@ def fp8_mm_grouped(a, b, a_scale, b_scale, c, row_offsets, variant=-1):
                                        offs, groups, n, k, variant, stream)
     if rc != RF_OK:
         raise RuntimeError("rf_fp8_gemm_grouped failed (%d): %s" % (rc, last_error()))
+
+
+def grouped_variant_for(row_offsets, n, k, num_cu=256):
+    """The tile form fp8_mm_grouped takes with variant=-1 for groups of these sizes on a device with num_cu compute
+    units (0..3: 256x256, 128x256, 128x128, 128x64 tiles; 4: 256-row tiles with a 128-row last tile; 5: the queue form).
+    Host arithmetic only."""
+    groups = len(row_offsets) - 1
+    offs = (ctypes.c_int32 * (groups + 1))(*[int(x) for x in row_offsets])
+    out = ctypes.c_int32(-1)
+    rc = lib().rf_grouped_variant_for(offs, groups, n, k, num_cu, ctypes.byref(out))
+    if rc != RF_OK:
+        raise RuntimeError("rf_grouped_variant_for failed (%d): %s" % (rc, last_error()))
+    return out.value
 
 
 def grouped_padded_offsets(row_offsets):

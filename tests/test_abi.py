@@ -6,6 +6,8 @@ import re
 import subprocess
 import sys
 
+import pytest
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
@@ -227,3 +229,33 @@ def test_planner_arithmetic_on_the_host_for_any_compute_unit_count(tmp_path):
     assert rfk.lib().rf_gemm_plan_for(16, 16, 100, 256, ctypes.byref(cfg)) == 1
     assert rfk.lib().rf_gemm_plan_for(16, 16, 128, 0, ctypes.byref(cfg)) == 1
     assert rfk.lib().rf_gemm_plan_for(16, 16, 128, 256, None) == 2
+
+
+def test_grouped_variant_choice_on_the_host():
+    """rf_grouped_variant_for needs no device. The queue form (5) is taken where its last tiles of 64..256 rows save at
+    least 7 % of the rows the other 256-wide forms compute and it has 1.5 items per compute unit (2.5 below K = 4096);
+    groups the other forms fit as well, or too few items, keep those forms; tiny problems take the form with the most
+    workgroups; bad arguments are refused."""
+    import numpy as np
+    import radeonflow_kernels_amd as rfk
+
+    def offs(sizes):
+        return [0] + [int(x) for x in np.cumsum(sizes)]
+
+    rng = np.random.default_rng(1)
+    cuts = np.sort(rng.choice(np.arange(1, 8192 // 16), 31, replace=False)) * 16
+    uneven = [0] + [int(x) for x in cuts] + [8192]                       # 32 groups of 16..816 rows
+    assert rfk.grouped_variant_for(uneven, 4096, 7168) == 5
+    assert rfk.grouped_variant_for(uneven, 4096, 7168, num_cu=304) == 5
+    assert rfk.grouped_variant_for(offs([256] * 32), 4096, 7168) in (0, 4)      # nothing to save
+    assert rfk.grouped_variant_for(offs([128] * 64), 4096, 7168) == 1
+    assert rfk.grouped_variant_for(offs([384] * 20), 4096, 7168) in (1, 4)
+    small = offs([int(x) * 16 for x in np.random.default_rng(5).integers(1, 25, 16)])    # 16 groups of 16..384 rows
+    assert rfk.grouped_variant_for(small, 2048, 7168) != 5              # 170 items for 256 units
+    assert rfk.grouped_variant_for(small, 7168, 7168) == 5              # the same groups, 3.5 times the column tiles
+    assert rfk.grouped_variant_for(uneven, 4096, 2048) == 5             # 816 items: 3.2 per unit
+    assert rfk.grouped_variant_for(uneven, 2048, 2048) != 5             # 408 items: 1.6 per unit, short items
+    assert rfk.grouped_variant_for(offs([64] * 8), 1024, 512) == 3      # no form fills the units: the most workgroups
+    for bad in (([0, 16, 8], 256, 256), ([1, 16], 256, 256), ([0, 16], 256, 100), ([0, 16], 0, 256)):
+        with pytest.raises(RuntimeError):
+            rfk.grouped_variant_for(*bad)

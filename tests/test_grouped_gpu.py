@@ -273,10 +273,12 @@ def test_grouped_queue_form_repeats_two_streams_and_graph_replays(rfk):
 
 
 def test_grouped_uneven_groups_take_the_queue_form_automatically(rfk):
-    """Uneven groups whose last tiles are much shorter than 128 rows: the automatic choice gives the bits of the queue
-    form and of every other form (all compute a row of C with the same operations in the same order)."""
-    rows = [16, 32, 272, 48, 528, 64, 16, 80, 304, 16, 32, 144, 16, 784, 48, 32, 16, 64, 272, 16]
-    g, offs, exp = _grouped_problem(rows, 2048, 256, seed=123, exact=True)
+    """Uneven groups whose last tiles are much shorter than 128 rows, enough of them for 2.5 items per compute unit: the
+    automatic choice is the queue form (rf_grouped_variant_for says so) and gives the bits of every other form (all
+    compute a row of C with the same operations in the same order)."""
+    rows = [16, 32, 272, 48, 528, 64, 16, 80, 304, 16, 32, 144, 16, 784, 48, 32, 16, 64, 272, 16] * 2
+    g, offs, exp = _grouped_problem(rows, 4096, 256, seed=123, exact=True)
+    assert rfk.grouped_variant_for(offs, 4096, 256, torch.cuda.get_device_properties(0).multi_processor_count) == 5
     for variant in (-1, 5, 1):
         g[4].zero_()
         rfk.fp8_mm_grouped(*g[:5], offs, variant=variant)
