@@ -708,3 +708,51 @@ def test_nan_codes_poison_their_row_or_column_only(rfk, m, n, k):
         got_nan = (got & 0x7FFF) > 0x7F80
         assert np.array_equal(got_nan, exp_nan), "NaN positions, plan %r" % (cfg,)
         assert np.array_equal(got[~exp_nan], exp[~exp_nan]), "plan %r" % (cfg,)
+
+
+def _random_operands(m, n, k, seed):
+    """fp8 codes 0..119 (finite, positive) and positive scales: rounding everywhere, no structure for a kernel to lean on"""
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    fp8 = torch.float8_e4m3fn
+    a = torch.randint(0, 120, (k, m), dtype=torch.uint8, device="cuda", generator=gen).view(fp8).T
+    b = torch.randint(0, 120, (k, n), dtype=torch.uint8, device="cuda", generator=gen).view(fp8).T
+    sa = (torch.rand((k // 128, m), device="cuda", generator=gen) * 1e-2).T
+    sb = (torch.rand((k // 128, (n + 127) // 128), device="cuda", generator=gen) * 1e-2).T
+    return a, b, sa, sb
+
+
+def _bits_under(rfk, ops, m, n, cfg):
+    c = torch.full((m, n), -3.0, dtype=torch.bfloat16, device="cuda")
+    rfk.fp8_mm(*ops, c, config=cfg)
+    torch.cuda.synchronize()
+    return bf16_bits(c)
+
+
+def test_skinny_k_schedule_on_random_shapes_equals_the_tile_kernel(rfk):
+    """40 seeded random shapes (M a multiple of 16 up to 8300, N a multiple of 64 up to 7600, K = 128 ... 512) with
+    rounding in every product: the skinny-K schedule gives the bits of the one-workgroup-per-tile kernel, twice."""
+    rng = np.random.default_rng(3)
+    for case in range(40):
+        m = int(rng.integers(1, 260)) * 16 if rng.random() < 0.7 else int(rng.integers(1, 520)) * 16
+        n = int(rng.integers(1, 65)) * 64 if rng.random() < 0.7 else int(rng.integers(1, 120)) * 64
+        k = int(rng.choice([128, 256, 384, 512]))
+        ops = _random_operands(m, n, k, case)
+        ref = _bits_under(rfk, ops, m, n, rfk.GemmConfig(1, 1, 8, 0))
+        for rep in range(2):
+            assert np.array_equal(_bits_under(rfk, ops, m, n, rfk.GemmConfig(0, 1, 8, 4)), ref), (m, n, k, rep)
+
+
+def test_k_split_inside_the_workgroup_on_random_shapes_equals_the_two_launch_form(rfk):
+    """30 seeded random shapes with an even number of K blocks: every variant that splits K between two wave groups
+    gives the bits of its one-group twin with split_k = 2 (partial sums through memory + reduction kernel)."""
+    rng = np.random.default_rng(7)
+    pairs = [(v["variant"], w["variant"]) for v in rfk.variants() if v["k_groups"] == 2 for w in rfk.variants()
+             if w["k_groups"] == 1 and (w["block_m"], w["block_n"], w["waves_m"], w["waves_n"]) ==
+             (v["block_m"], v["block_n"], v["waves_m"], v["waves_n"]) and 0 <= v["lds_bytes"] - 2 * w["lds_bytes"] < 4096]
+    assert len(pairs) >= 2
+    for case in range(30):
+        m, n, k = int(rng.integers(1, 130)) * 16, int(rng.integers(1, 200)) * 16, int(rng.integers(1, 30)) * 256
+        ops = _random_operands(m, n, k, 100 + case)
+        for v, twin in pairs:
+            ref = _bits_under(rfk, ops, m, n, rfk.GemmConfig(twin, 2, 8, 0))
+            assert np.array_equal(_bits_under(rfk, ops, m, n, rfk.GemmConfig(v, 1, 8, 0)), ref), (v, m, n, k)

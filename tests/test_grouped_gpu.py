@@ -285,3 +285,35 @@ def test_grouped_uneven_groups_take_the_queue_form_automatically(rfk):
         torch.cuda.synchronize()
         assert np.array_equal(bf16_bits(g[4]), exp), "variant %d" % variant
     _check_canary(g[5], g[4].numel())
+
+
+def test_grouped_queue_form_on_random_layouts_equals_the_128_row_tiles(rfk):
+    """60 seeded random layouts (1 to 256 groups of 0 to 700 rows, half of them with sizes that are not multiples of 16;
+    N = 256 ... 4096, K = 128 ... 1024) with rounding in every product: the queue form, the queue form again and the
+    automatic choice give the bits of the 128 x 256 tiles, and rows of C outside the groups' rows keep their fill."""
+    rng = np.random.default_rng(1)
+    fp8 = torch.float8_e4m3fn
+    for case in range(60):
+        groups = int(rng.choice([1, 2, 3, 5, 8, 13, 16, 17, 31, 64, 100, 200, 256]))
+        hi = int(rng.choice([20, 70, 130, 300, 700]))
+        sizes = [int(x) for x in rng.integers(0, hi + 1, groups)]
+        if rng.random() < 0.5:
+            sizes = [s // 16 * 16 for s in sizes]
+        if sum(sizes) == 0:
+            sizes[0] = 16
+        n, k = int(rng.choice([256, 272, 512, 768, 1024, 1536, 2048, 4096])), int(rng.choice([128, 256, 384, 512, 1024]))
+        offs = [0] + [int(x) for x in np.cumsum(sizes)]
+        gm = offs[-1]
+        gen = torch.Generator(device="cuda").manual_seed(case)
+        a = torch.randint(0, 120, (k, gm), dtype=torch.uint8, device="cuda", generator=gen).view(fp8).T
+        b = torch.randint(0, 120, (groups, k, n), dtype=torch.uint8, device="cuda", generator=gen).view(fp8).permute(0, 2, 1)
+        sa = (torch.rand((k // 128, gm), device="cuda", generator=gen) * 1e-2).T
+        sb = (torch.rand((groups, k // 128, (n + 127) // 128), device="cuda", generator=gen) * 1e-2).permute(0, 2, 1)
+        outs = []
+        for variant in (1, 5, 5, -1):
+            c = torch.full((gm, n), -3.0, dtype=torch.bfloat16, device="cuda")
+            rfk.fp8_mm_grouped(a, b, sa, sb, c, offs, variant=variant)
+            torch.cuda.synchronize()
+            outs.append(bf16_bits(c))
+        for o in outs[1:]:
+            assert np.array_equal(outs[0], o), (case, groups, n, k, sizes[:12])
